@@ -27,7 +27,7 @@ __global__ void embed_gather_kernel(const TT* __restrict__ table, const int* __r
 // between `block` gate columns and the `block` matching up columns (gate is its first column).
 template <typename T>
 __global__ void silu_mul_kernel(const T* __restrict__ gate, const T* __restrict__ up,
-                                int64_t in_stride, T* __restrict__ out, int width, int block) {
+                                int64_t in_stride, T* __restrict__ out, int width, int block, int act_code) {
   const int t = blockIdx.x;
   const int j = blockIdx.y * blockDim.x + threadIdx.x;
   if (j >= width) return;
@@ -35,7 +35,7 @@ __global__ void silu_mul_kernel(const T* __restrict__ gate, const T* __restrict_
   const int64_t gi = block > 0 ? row + (j / block) * 2 * block + j % block : row + j;
   const float g = to_float(gate[gi]);
   const float u = to_float(block > 0 ? gate[gi + block] : up[gi]);
-  const float act = g / (1.0f + expf(-g));
+  const float act = gate_act(g, act_code);
   out[static_cast<int64_t>(t) * width + j] = from_float<T>(act * u);
 }
 
@@ -43,7 +43,7 @@ __global__ void silu_mul_kernel(const T* __restrict__ gate, const T* __restrict_
 // in_stride are multiples of 8 and the pointers 16-byte aligned (the launcher checks).
 __global__ void silu_mul_bf16x8_kernel(const uint16_t* __restrict__ gate, const uint16_t* __restrict__ up,
                                        int64_t in_stride, uint16_t* __restrict__ out, int width, int block,
-                                       int64_t chunks) {
+                                       int64_t chunks, int act_code) {
   const int64_t c = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (c >= chunks) return;
   const int per_row = width / 8;
@@ -59,7 +59,7 @@ __global__ void silu_mul_bf16x8_kernel(const uint16_t* __restrict__ gate, const 
   for (int i = 0; i < 4; ++i) {
     const float g0 = __uint_as_float(gw[i] << 16), g1 = __uint_as_float(gw[i] & 0xffff0000u);
     const float u0 = __uint_as_float(uw[i] << 16), u1 = __uint_as_float(uw[i] & 0xffff0000u);
-    ow[i] = pack_bf16x2(g0 / (1.0f + expf(-g0)) * u0, g1 / (1.0f + expf(-g1)) * u1);
+    ow[i] = pack_bf16x2(gate_act(g0, act_code) * u0, gate_act(g1, act_code) * u1);
   }
   *reinterpret_cast<uint4*>(out + t * width + j) = uint4{ow[0], ow[1], ow[2], ow[3]};
 }
@@ -123,8 +123,9 @@ extern "C" int arle_embed_gather(const void* table, int table_dtype, const int* 
 
 // gate and up are two columns blocks of rows with a common row stride (in
 // elements), so one fused [T, 2I] buffer and two separate buffers both fit.
-extern "C" int arle_silu_mul(const void* gate, const void* up, long long in_stride, void* out,
-                             int dtype, int tokens, int width, int block, void* stream) {
+// act: kActSilu or kActGeluTanh.
+extern "C" int arle_act_mul(const void* gate, const void* up, long long in_stride, void* out,
+                            int dtype, int tokens, int width, int block, int act, void* stream) {
   if (tokens == 0 || width == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
@@ -133,20 +134,25 @@ extern "C" int arle_silu_mul(const void* gate, const void* up, long long in_stri
     const int64_t chunks = static_cast<int64_t>(tokens) * (width / 8);
     silu_mul_bf16x8_kernel<<<static_cast<unsigned>((chunks + 255) / 256), 256, 0, s>>>(
         static_cast<const uint16_t*>(gate), static_cast<const uint16_t*>(up), in_stride,
-        static_cast<uint16_t*>(out), width, block, chunks);
+        static_cast<uint16_t*>(out), width, block, chunks, act);
     return launch_status();
   }
   dim3 grid(tokens, (width + 255) / 256);
   if (dtype == kF32) {
     silu_mul_kernel<float><<<grid, 256, 0, s>>>(static_cast<const float*>(gate),
                                                 static_cast<const float*>(up), in_stride,
-                                                static_cast<float*>(out), width, block);
+                                                static_cast<float*>(out), width, block, act);
   } else {
     silu_mul_kernel<bf16><<<grid, 256, 0, s>>>(static_cast<const bf16*>(gate),
                                                static_cast<const bf16*>(up), in_stride,
-                                               static_cast<bf16*>(out), width, block);
+                                               static_cast<bf16*>(out), width, block, act);
   }
   return launch_status();
+}
+
+extern "C" int arle_silu_mul(const void* gate, const void* up, long long in_stride, void* out,
+                             int dtype, int tokens, int width, int block, void* stream) {
+  return arle_act_mul(gate, up, in_stride, out, dtype, tokens, width, block, kActSilu, stream);
 }
 
 // parts [n_parts][count] float32 (stride elements apart) -> out [count] float32 or bfloat16.

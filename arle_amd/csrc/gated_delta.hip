@@ -1,0 +1,199 @@
+// The gated delta rule, token by token, for the rows of a packed step, continued across steps through a
+// per-request state S [heads, D, Dv] in 32-bit floats.
+//
+// Per head, with q and k of D entries (head h reads q/k head h / (H / G)) and v of Dv:
+//   q <- q / sqrt(sum q^2 + 1e-6) * D^(-1/2),   k <- k / sqrt(sum k^2 + 1e-6)
+//   beta = sigmoid(b),   g = exp(-exp(A_log_h) * softplus(a + dt_bias_h))
+//   S <- g S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q
+// A column of S (one entry of v) never meets another, so the columns spread over workgroups: a workgroup a
+// (request, head, 16 columns), four columns a wave, a sixteenth of D a lane.  Rows go through LDS in blocks of
+// 32; the block's unit norms, gates and the dot products k . q are made there, a row by eight threads, always
+// the same entries in the same order.  The chain of a row is one pass over the lane's share of the old S for both
+// S^T k and S^T q (o = g S_old^T q + u (k . q), which is S_new^T q), one exchange over the sixteen shares, and the
+// update.  `gated_delta_output` divides each head's o by its root mean square, multiplies by the norm's weight and
+// by silu of the gate's projection.
+#include "common.h"
+
+namespace arle {
+
+constexpr int kGdWaves = 4;
+constexpr int kGdThreads = kGdWaves * kWave;
+constexpr int kGdWaveCols = 4;
+constexpr int kGdParts = kWave / kGdWaveCols;     // shares of D
+constexpr int kGdCols = kGdWaves * kGdWaveCols;   // columns of a workgroup
+constexpr int kGdRows = 32;                       // rows staged at a time
+constexpr int kGdRowThreads = kGdThreads / kGdRows;   // threads that prepare a row
+
+__device__ __forceinline__ float softplus(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
+
+template <typename T, int DS>
+__global__ __launch_bounds__(kGdThreads) void gated_delta_scan_kernel(
+    const T* __restrict__ q, long long q_stride, const T* __restrict__ k, long long k_stride, const T* __restrict__ v,
+    long long v_stride, const float* __restrict__ gates /* [T, >= 2H]: b then a */, long long gates_stride,
+    const float* __restrict__ a_log, const float* __restrict__ dt_bias, float unit_eps, float* __restrict__ s_state,
+    const int* __restrict__ seg_row0, const int* __restrict__ seg_slot, float* __restrict__ out /* [T, H * Dv] */,
+    int H, int G, int D, int Dv) {
+  constexpr int DP = kGdParts * DS;   // padded D: what lies past D is zero in LDS and in the registers
+  __shared__ __attribute__((aligned(16))) float q_lds[kGdRows][DP];
+  __shared__ __attribute__((aligned(16))) float k_lds[kGdRows][DP];
+  __shared__ float v_lds[kGdRows][kGdCols];
+  __shared__ float c_lds[kGdRows][4];   // decay, beta, k . q
+  const int seg = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int lane = tid % kWave, wave = tid / kWave;
+  const int kvh = h / (H / G);
+  const int col_in = wave * kGdWaveCols + lane % kGdWaveCols;
+  const int col = blockIdx.z * kGdCols + col_in;
+  const int part = lane / kGdWaveCols;
+  const bool live = col < Dv;
+  const int row0 = seg_row0[seg], rows = seg_row0[seg + 1] - row0;
+  float* s_ptr = s_state + (static_cast<int64_t>(seg_slot[seg]) * H + h) * D * Dv;
+  const float rate = expf(a_log[h]), bias = dt_bias[h], q_scale = 1.0f / sqrtf(static_cast<float>(D));
+
+  float S[DS];
+#pragma unroll
+  for (int i = 0; i < DS; ++i) {
+    const int d = part * DS + i;
+    S[i] = (live && d < D) ? s_ptr[static_cast<int64_t>(d) * Dv + col] : 0.f;
+  }
+  for (int base = 0; base < rows; base += kGdRows) {
+    const int n = min(kGdRows, rows - base);
+    __syncthreads();   // the block before has been read
+    {   // a row by kGdRowThreads threads: its q and k to LDS, their unit norms, k . q, the gates
+      const int r = tid / kGdRowThreads, sub = tid % kGdRowThreads;
+      const int64_t t = row0 + base + min(r, n - 1);
+      const T* qr = q + t * q_stride + kvh * D;
+      const T* kr = k + t * k_stride + kvh * D;
+      float sq = 0.f, sk = 0.f, kq = 0.f;
+      for (int d = sub; d < DP; d += kGdRowThreads) {
+        const float qv = d < D ? to_float(qr[d]) : 0.f, kv = d < D ? to_float(kr[d]) : 0.f;
+        q_lds[r][d] = qv;
+        k_lds[r][d] = kv;
+        sq = fmaf(qv, qv, sq);
+        sk = fmaf(kv, kv, sk);
+        kq = fmaf(kv, qv, kq);
+      }
+#pragma unroll
+      for (int off = kGdRowThreads / 2; off > 0; off >>= 1) {
+        sq += __shfl_xor(sq, off, kWave);
+        sk += __shfl_xor(sk, off, kWave);
+        kq += __shfl_xor(kq, off, kWave);
+      }
+      const float fq = q_scale / sqrtf(sq + unit_eps), fk = 1.0f / sqrtf(sk + unit_eps);
+      for (int d = sub; d < DP; d += kGdRowThreads) {   // the entries this thread has written itself
+        q_lds[r][d] *= fq;
+        k_lds[r][d] *= fk;
+      }
+      if (sub == 0) {
+        const float b = gates[t * gates_stride + h], a = gates[t * gates_stride + H + h];
+        c_lds[r][0] = expf(-rate * softplus(a + bias));
+        c_lds[r][1] = 1.0f / (1.0f + expf(-b));
+        c_lds[r][2] = kq * fq * fk;
+      }
+      for (int e = tid; e < kGdRows * kGdCols; e += kGdThreads) {
+        const int rr = e / kGdCols, cc = e % kGdCols;
+        const int64_t tt = row0 + base + min(rr, n - 1);
+        const int c_abs = min(static_cast<int>(blockIdx.z) * kGdCols + cc, Dv - 1);
+        v_lds[rr][cc] = to_float(v[tt * v_stride + h * Dv + c_abs]);
+      }
+    }
+    __syncthreads();
+    for (int r = 0; r < n; ++r) {
+      const float g = c_lds[r][0], beta = c_lds[r][1], kq = c_lds[r][2];
+      float kk[DS], dk = 0.f, dq = 0.f;
+      if constexpr (DS % 4 == 0) {
+        const float4* k4 = reinterpret_cast<const float4*>(&k_lds[r][part * DS]);
+        const float4* q4 = reinterpret_cast<const float4*>(&q_lds[r][part * DS]);
+#pragma unroll
+        for (int i = 0; i < DS / 4; ++i) {
+          const float4 kv = k4[i], qv = q4[i];
+          kk[4 * i] = kv.x; kk[4 * i + 1] = kv.y; kk[4 * i + 2] = kv.z; kk[4 * i + 3] = kv.w;
+          dq = fmaf(S[4 * i], qv.x, dq); dq = fmaf(S[4 * i + 1], qv.y, dq);
+          dq = fmaf(S[4 * i + 2], qv.z, dq); dq = fmaf(S[4 * i + 3], qv.w, dq);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < DS; ++i) {
+          kk[i] = k_lds[r][part * DS + i];
+          dq = fmaf(S[i], q_lds[r][part * DS + i], dq);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < DS; ++i) dk = fmaf(S[i], kk[i], dk);
+#pragma unroll
+      for (int off = kGdWaveCols; off < kWave; off <<= 1) {   // over the shares of D, in a fixed order
+        dk += __shfl_xor(dk, off, kWave);
+        dq += __shfl_xor(dq, off, kWave);
+      }
+      const float u = beta * (v_lds[r][col_in] - g * dk);
+#pragma unroll
+      for (int i = 0; i < DS; ++i) S[i] = fmaf(kk[i], u, g * S[i]);
+      if (part == 0 && live) out[static_cast<int64_t>(row0 + base + r) * (H * Dv) + h * Dv + col] = fmaf(u, kq, g * dq);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < DS; ++i) {
+    const int d = part * DS + i;
+    if (live && d < D) s_ptr[static_cast<int64_t>(d) * Dv + col] = S[i];
+  }
+}
+
+// One wave a (row, head): o / rms(o) * w * silu(gate).
+template <typename T>
+__global__ __launch_bounds__(kWave) void gated_delta_output_kernel(const float* __restrict__ o, const T* __restrict__ gate,
+                                                                   long long gate_stride, const void* __restrict__ weight,
+                                                                   int w_dtype, float eps, T* __restrict__ out, int H,
+                                                                   int Dv) {
+  const int64_t t = blockIdx.x;
+  const int h = blockIdx.y, lane = threadIdx.x;
+  const float* row = o + (t * H + h) * Dv;
+  float ss = 0.f;
+  for (int d = lane; d < Dv; d += kWave) ss = fmaf(row[d], row[d], ss);
+  const float inv = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(Dv) + eps);
+  for (int d = lane; d < Dv; d += kWave) {
+    const float z = to_float(gate[t * gate_stride + h * Dv + d]);
+    out[(t * H + h) * Dv + d] = from_float<T>(row[d] * inv * load_as_float(weight, w_dtype, d) * (z / (1.0f + expf(-z))));
+  }
+}
+
+}  // namespace arle
+
+using namespace arle;
+
+extern "C" int arle_gated_delta_scan(const void* q, long long q_stride, const void* k, long long k_stride, const void* v,
+                                     long long v_stride, int dtype, const void* gates, long long gates_stride,
+                                     const void* a_log, const void* dt_bias, float unit_eps, void* s_state,
+                                     const int* seg_row0, const int* seg_slot, int segments, void* out, int H, int G,
+                                     int D, int Dv, void* stream) {
+  if (segments == 0) return 0;
+  if (D < 1 || D > 256 || H % G) return static_cast<int>(hipErrorInvalidValue);
+  dim3 grid(segments, H, (Dv + kGdCols - 1) / kGdCols);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define ARLE_GD(T, DS)                                                                                               \
+  gated_delta_scan_kernel<T, DS><<<grid, kGdThreads, 0, s>>>(                                                        \
+      static_cast<const T*>(q), q_stride, static_cast<const T*>(k), k_stride, static_cast<const T*>(v), v_stride,    \
+      static_cast<const float*>(gates), gates_stride, static_cast<const float*>(a_log),                              \
+      static_cast<const float*>(dt_bias), unit_eps, static_cast<float*>(s_state), seg_row0, seg_slot,                \
+      static_cast<float*>(out), H, G, D, Dv)
+#define ARLE_GD_T(T)                                                                                                 \
+  if (D <= 32) ARLE_GD(T, 2); else if (D <= 64) ARLE_GD(T, 4); else if (D <= 128) ARLE_GD(T, 8); else ARLE_GD(T, 16)
+  if (dtype == kF32) { ARLE_GD_T(float); } else { ARLE_GD_T(bf16); }
+#undef ARLE_GD_T
+#undef ARLE_GD
+  return launch_status();
+}
+
+extern "C" int arle_gated_delta_output(const void* o, const void* gate, long long gate_stride, int dtype,
+                                       const void* weight, int w_dtype, float eps, void* out, int tokens, int H, int Dv,
+                                       void* stream) {
+  if (tokens == 0) return 0;
+  dim3 grid(tokens, H);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == kF32) {
+    gated_delta_output_kernel<float><<<grid, kWave, 0, s>>>(static_cast<const float*>(o), static_cast<const float*>(gate),
+                                                            gate_stride, weight, w_dtype, eps, static_cast<float*>(out), H, Dv);
+  } else {
+    gated_delta_output_kernel<bf16><<<grid, kWave, 0, s>>>(static_cast<const float*>(o), static_cast<const bf16*>(gate),
+                                                           gate_stride, weight, w_dtype, eps, static_cast<bf16*>(out), H, Dv);
+  }
+  return launch_status();
+}

@@ -2,6 +2,7 @@
 // steps through a per-request state of the last taps-1 inputs.
 //
 //   y_t[c] = (ADD ? u_t[c] : 0) + sum_{j < taps} w[c][j] * u_(t - taps + 1 + j)[c],    u := input (+ bias)
+//   (SILU: y <- y / (1 + exp(-y)) on the way out.  The entry point's `add_input` holds both: bit 0 ADD, bit 1 SILU.)
 //
 // The rows of one request are consecutive in the step; an input further back than the request's first row of
 // this step comes from its state [slots][taps-1][channels] (the most recent input last), which is all zeros
@@ -13,6 +14,9 @@
 namespace arle {
 
 constexpr int kConvMaxTaps = 16;
+constexpr int kConvAdd = 1, kConvSilu = 2;
+
+__device__ __forceinline__ float conv_out(float y, int flags) { return (flags & kConvSilu) ? y / (1.0f + expf(-y)) : y; }
 
 __global__ void causal_conv_kernel(const void* __restrict__ u, long long u_stride, int u_dtype,
                                    const void* __restrict__ bias, int bias_dtype, const void* __restrict__ w,
@@ -32,7 +36,7 @@ __global__ void causal_conv_kernel(const void* __restrict__ u, long long u_strid
   // rows of the same request right before this one in the step (at most taps-1 matter)
   int mine = 0;
   while (mine < taps - 1 && t - mine - 1 >= 0 && slot_of_token[t - mine - 1] == slot) ++mine;
-  float acc = add_input ? now : 0.f;
+  float acc = (add_input & kConvAdd) ? now : 0.f;
   acc = fmaf(load_as_float(w, w_dtype, static_cast<int64_t>(c) * taps + taps - 1), now, acc);
   for (int back = 1; back < taps; ++back) {
     float v;
@@ -44,7 +48,7 @@ __global__ void causal_conv_kernel(const void* __restrict__ u, long long u_strid
     }
     acc = fmaf(load_as_float(w, w_dtype, static_cast<int64_t>(c) * taps + taps - 1 - back), v, acc);
   }
-  store_from_float(out, out_dtype, t * out_stride + c, acc);
+  store_from_float(out, out_dtype, t * out_stride + c, conv_out(acc, add_input));
 }
 
 // One element type T throughout and channels in whole groups of four: a lane takes four channels of a row with one
@@ -84,14 +88,15 @@ __global__ void causal_conv_vec_kernel(const T* __restrict__ u, long long u_stri
   float acc[4];
   const float now[4] = {in[0].x, in[0].y, in[0].z, in[0].w};
 #pragma unroll
-  for (int i = 0; i < 4; ++i) acc[i] = fmaf(wt[i][TAPS - 1], now[i], add_input ? now[i] : 0.f);
+  for (int i = 0; i < 4; ++i) acc[i] = fmaf(wt[i][TAPS - 1], now[i], (add_input & kConvAdd) ? now[i] : 0.f);
 #pragma unroll
   for (int back = 1; back < TAPS; ++back) {
     const float v[4] = {in[back].x, in[back].y, in[back].z, in[back].w};
 #pragma unroll
     for (int i = 0; i < 4; ++i) acc[i] = fmaf(wt[i][TAPS - 1 - back], v[i], acc[i]);
   }
-  st4<T>(out + t * out_stride + c, float4{acc[0], acc[1], acc[2], acc[3]});
+  st4<T>(out + t * out_stride + c, float4{conv_out(acc[0], add_input), conv_out(acc[1], add_input), conv_out(acc[2], add_input),
+                                         conv_out(acc[3], add_input)});
 }
 
 // One thread a (segment, channel): the new state is the last taps-1 of (old state, this step's inputs).

@@ -42,6 +42,9 @@ SOURCES = {
     "post_norm": "post_norm.hip",
     "latent": "latent.hip",
     "moe": "moe.hip",
+    "hyper": "hyper.hip",
+    "rotary_store": "rotary_store.hip",
+    "gated_delta": "gated_delta.hip",
     "host": "host/runtime.cpp",
 }
 HEADERS = ("common.h", "attention_static.h", "attention_args.h", "attention_stream.h", "attention_portions.h",

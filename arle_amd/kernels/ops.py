@@ -1352,13 +1352,16 @@ def run_product(choice: ProductChoice, x, w, tiles, out_dtype, partials_ok: bool
     return out
 
 
-def gate_up_act(x: torch.Tensor, w: torch.Tensor, tiles: torch.Tensor | None = None) -> torch.Tensor:
-    """silu(x . gate^T) * (x . up^T) for w [2I, K] holding gate and up rows interleaved in blocks of 16: [M, I]."""
+def gate_up_act(x: torch.Tensor, w: torch.Tensor, tiles: torch.Tensor | None = None, act: int = 0) -> torch.Tensor:
+    """act(x . gate^T) * (x . up^T) for w [2I, K] holding gate and up rows interleaved in blocks of 16: [M, I];
+    act 0: silu, 1: the tanh form of gelu."""
     _gpu(x, w)
     _rows(x, "x")
     rows, n, k = x.shape[0], w.shape[0], x.shape[1]
     if rows == 0:
         return torch.empty((0, n // 2), dtype=x.dtype, device=x.device)
+    if act != 0:     # the products that apply the activation themselves know silu only
+        return act_mul_interleaved(gemm_bf16(x, w, x.dtype, tiles=tiles), act, 16)
     choice = choose_product(rows, n, k, x.stride(0), tiled=tiles is not None, fused=True, partials_ok=False,
                             aligned=x.data_ptr() % 16 == 0)
     return run_product(choice, x, w, tiles, x.dtype, False, fused=True)
@@ -1443,10 +1446,11 @@ CONV_MAX_TAPS = 16
 
 
 def causal_conv(u: torch.Tensor, weight, state, slot_of_token: torch.Tensor, *, bias=None, add_input: bool = False,
-                out_dtype: torch.dtype | None = None):
+                out_dtype: torch.dtype | None = None, silu: bool = False):
     """y_t = (u_t if add_input) + sum_j weight[:, j] * u_(t - taps + 1 + j) per channel, over the rows of each request
     (consecutive in u) and, further back, over its state [slots, taps-1, C]; u counts with `bias` added.  weight
-    None: y = u + bias.  The state is not changed: `conv_state_update` does that once the step's rows are done."""
+    None: y = u + bias.  silu: y / (1 + exp(-y)) is what comes out.  The state is not changed: `conv_state_update`
+    does that once the step's rows are done."""
     _gpu(u, weight, state, slot_of_token, bias)
     _rows(u, "u")
     tokens, channels = u.shape
@@ -1467,7 +1471,7 @@ def causal_conv(u: torch.Tensor, weight, state, slot_of_token: torch.Tensor, *, 
     lib.call("arle_causal_conv", u.data_ptr(), u.stride(0), _code(u), _ptr(bias), _code(bias) if bias is not None else 0,
              _ptr(weight), _code(weight) if weight is not None else 0, state.data_ptr() if has_state else 0,
              _code(state) if has_state else 0, slot_of_token.data_ptr(), out.data_ptr(), out.stride(0), _code(out),
-             tokens, channels, taps, 1 if add_input else 0, _stream())
+             tokens, channels, taps, (1 if add_input else 0) | (2 if silu else 0), _stream())
     return out
 
 
@@ -1934,4 +1938,213 @@ def moe_expert(x, w, ids, *, gate_up: bool):
     out = torch.empty((tokens * top, N), dtype=x.dtype if gate_up else torch.float32, device=x.device)
     lib.call("arle_moe_expert", x.data_ptr(), x.stride(0), w.data_ptr(), ids.data_ptr(), out.data_ptr(), _code(x),
              1 if gate_up else 0, tokens, w.shape[0], top, N, x.shape[1], _stream())
+    return out
+
+
+# ------------------------------------------------------------- gated feed-forward activations
+
+ACT_SILU, ACT_GELU_TANH = 0, 1
+ACTIVATIONS = {"silu": ACT_SILU, "gelu_tanh": ACT_GELU_TANH}
+
+
+def act_mul(gate: torch.Tensor, up: torch.Tensor, act: int = ACT_SILU):
+    """out = act(gate) * up for two [T, I] views with the same row stride; act: ACT_SILU or ACT_GELU_TANH
+    (0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))))."""
+    _gpu(gate, up)
+    _rows(gate, "gate")
+    _rows(up, "up")
+    _need(gate.shape == up.shape and gate.dtype == up.dtype and gate.stride(0) == up.stride(0),
+          "gate and up must agree in shape, dtype and row stride")
+    _need(act in (ACT_SILU, ACT_GELU_TANH), "unknown activation code")
+    tokens, width = gate.shape
+    _need(math.ceil(width / 256) <= _GRID_Y_MAX, "act_mul: width too large")
+    out = torch.empty((tokens, width), dtype=gate.dtype, device=gate.device)
+    lib.call("arle_act_mul", gate.data_ptr(), up.data_ptr(), gate.stride(0), out.data_ptr(), _code(gate), tokens, width,
+             0, int(act), _stream())
+    return out
+
+
+def act_mul_interleaved(gate_up: torch.Tensor, act: int = ACT_SILU, block: int = 16):
+    """`act_mul` for a [T, 2I] buffer whose columns alternate between `block` gate columns and the matching up columns."""
+    _gpu(gate_up)
+    _rows(gate_up, "gate_up")
+    tokens, two_i = gate_up.shape
+    _need(block > 0 and two_i % (2 * block) == 0, "interleaved gate/up width must be a multiple of 2*block")
+    width = two_i // 2
+    _need(math.ceil(width / 256) <= _GRID_Y_MAX, "act_mul: width too large")
+    out = torch.empty((tokens, width), dtype=gate_up.dtype, device=gate_up.device)
+    lib.call("arle_act_mul", gate_up.data_ptr(), gate_up.data_ptr(), gate_up.stride(0), out.data_ptr(), _code(gate_up),
+             tokens, width, int(block), int(act), _stream())
+    return out
+
+
+# ------------------------------------------------------- residual streams with learned connections
+
+HYPER_MAX_STREAMS = 16
+HYPER_MAX_WIDTH = 16000
+
+
+def _stack_args(y, rows: int, width: int, name: str):
+    """(pointer, type code, row stride, parts, part stride) of a sublayer's output: a tensor [T, W] of a kernel type
+    or a contiguous float32 stack [P, T, W] of partial sums."""
+    if y.dim() == 3:
+        _need(y.dtype == torch.float32 and y.is_contiguous() and tuple(y.shape[1:]) == (rows, width) and y.shape[0] >= 1,
+              f"{name}: a stack of partial sums must be contiguous float32 [P, T, W]")
+        return y.data_ptr(), F32, width, y.shape[0], rows * width
+    _rows(y, name)
+    _need(y.shape == (rows, width) and y.dtype in _CODES, f"{name} must be [T, W]")
+    return y.data_ptr(), _code(y), y.stride(0), 1, 0
+
+
+def hyper_step(streams: torch.Tensor, y, mix, out_w, in_w, norm_w: torch.Tensor, eps: float, out_dtype: torch.dtype, *,
+               num_streams: int, rows=None):
+    """One step of a residual of `num_streams` streams (see csrc/hyper.hip): write the output y of the sublayer before
+    through its connection (mix [S, S] indexed [from, to], out_w [S]; y None: nothing to write), then read through the
+    next sublayer's connection (in_w [S]; None: the plain sum) and RMS-norm with norm_w.
+
+    streams: float32 [T, S, W], updated in place, or float32 [T, W] (every stream starts as a copy of it; a new
+    [T, S, W] tensor is made).  rows (int32 [R]): only these tokens are read, nothing is written.  Returns
+    (streams [T, S, W], normed [T or R, W] in out_dtype)."""
+    _gpu(streams, y, mix, out_w, in_w, norm_w, rows)
+    S = int(num_streams)
+    _need(1 <= S <= HYPER_MAX_STREAMS, f"1..{HYPER_MAX_STREAMS} streams")
+    _need(streams.dtype == torch.float32 and streams.is_contiguous() and streams.dim() in (2, 3),
+          "streams must be contiguous float32 [T, S, W] or [T, W]")
+    tokens, width = streams.shape[0], streams.shape[-1]
+    _need(0 < width <= HYPER_MAX_WIDTH, f"hyper_step takes widths up to {HYPER_MAX_WIDTH}")
+    if streams.dim() == 3:
+        _need(streams.shape[1] == S, "streams must be [T, S, W]")
+        src_strides, dst = (S * width, width), streams
+    else:
+        src_strides = (width, 0)
+        dst = streams if rows is not None else torch.empty((tokens, S, width), dtype=torch.float32, device=streams.device)
+    for name, t, shape in (("mix", mix, (S, S)), ("out_w", out_w, (S,)), ("in_w", in_w, (S,)), ("norm_w", norm_w, (width,))):
+        if t is not None:
+            _need(tuple(t.shape) == shape and t.dtype == torch.float32 and t.is_contiguous(), f"{name} must be float32 {shape}")
+    y_args = (0, 0, 0, 0, 0)
+    if y is not None:
+        _need(mix is not None and out_w is not None, "an output is written through a connection")
+        y_args = _stack_args(y, tokens, width, "y")
+    grid = tokens
+    if rows is not None:
+        _i32(rows, "rows")
+        grid = rows.numel()
+    out = torch.empty((grid, width), dtype=out_dtype, device=streams.device)
+    vec = (width % 4 == 0 and (y is None or (y_args[2] % 4 == 0 and y_args[0] % 16 == 0)))
+    lib.call("arle_hyper_step", streams.data_ptr(), src_strides[0], src_strides[1],
+             0 if rows is not None else dst.data_ptr(), *y_args, _ptr(mix), _ptr(out_w), _ptr(in_w), norm_w.data_ptr(),
+             float(eps), _ptr(rows), out.data_ptr(), _CODES[out_dtype], width, grid, S, width, 1 if vec else 0, _stream())
+    return dst, out
+
+
+def pair_norm(a, b, weight_a, weight_b, eps: float, coef: float = 0.5):
+    """float32 [T, W]: coef * (a / rms(a) * weight_a + b / rms(b) * weight_b), rms over W with eps inside the root;
+    a and b are tensors [T, W] of one type or float32 stacks [P, T, W] of partial sums."""
+    _gpu(a, b, weight_a, weight_b)
+    tokens, width = a.shape[-2], a.shape[-1]
+    if a.dtype != b.dtype:
+        a, b = a.float(), b.float()
+    pa, ca, sa, na, nsa = _stack_args(a, tokens, width, "a")
+    pb, cb, sb, nb, nsb = _stack_args(b, tokens, width, "b")
+    for w in (weight_a, weight_b):
+        _need(w.shape == (width,) and w.dtype == torch.float32 and w.is_contiguous(), "the weights must be float32 [W]")
+    out = torch.empty((tokens, width), dtype=torch.float32, device=a.device)
+    vec = width % 4 == 0 and sa % 4 == 0 and sb % 4 == 0 and pa % 16 == 0 and pb % 16 == 0
+    lib.call("arle_pair_norm", pa, sa, na, nsa, pb, sb, nb, nsb, ca, weight_a.data_ptr(), weight_b.data_ptr(), float(eps),
+             float(coef), out.data_ptr(), tokens, width, 1 if vec else 0, _stream())
+    return out
+
+
+# ------------------------------------------------------ attention operands with rotary positions
+
+ROTARY_MAX_HEAD_DIM = 1024
+
+
+def rotary_qkv_store(q, k, v, *, num_q_heads: int, num_kv_heads: int, key_dim: int, value_dim: int, eps: float,
+                     q_weight=None, k_weight=None, unit_after: bool = False, cos=None, sin=None, rotary_dim: int = 0,
+                     interleaved: bool = False, positions, slot_of_token, block_table, k_pages, v_pages, page_size: int):
+    """Per head of q (in place) and k (to the pages): an RMS norm with a weight [Dk] in front of the rotation
+    (q_weight, k_weight given), the rotation of the first `rotary_dim` entries by the angles of float32 tables
+    cos, sin [positions, rotary_dim / 2] (pairs (i, i + rotary_dim / 2), or (2i, 2i + 1) if `interleaved`), and a
+    division by the root mean square behind it (`unit_after`); v goes to the pages as it is."""
+    _gpu(q, k, v, q_weight, k_weight, cos, sin, positions, slot_of_token, block_table, k_pages, v_pages)
+    tokens = q.shape[0]
+    for name, t, width in (("q", q, num_q_heads * key_dim), ("k", k, num_kv_heads * key_dim), ("v", v, num_kv_heads * value_dim)):
+        _rows(t, name)
+        _need(t.shape == (tokens, width) and t.dtype == q.dtype and t.dtype in _CODES, f"{name} must be [T, {width}]")
+    _need(0 < key_dim <= ROTARY_MAX_HEAD_DIM and value_dim > 0 and num_q_heads + 2 * num_kv_heads <= _GRID_Y_MAX,
+          "head sizes or counts out of range")
+    _need((q_weight is None) == (k_weight is None), "give both norm weights or neither")
+    w_code = 0
+    if q_weight is not None:
+        for w in (q_weight, k_weight):
+            _need(w.shape == (key_dim,) and w.is_contiguous() and w.dtype in _CODES, "a q/k norm weight must be [Dk]")
+        _need(q_weight.dtype == k_weight.dtype, "q and k norm weights must be of one type")
+        w_code = _code(q_weight)
+    _need(0 <= rotary_dim <= key_dim and rotary_dim % 2 == 0, "rotary_dim must be even and at most the key size")
+    if rotary_dim:
+        for name, t in (("cos", cos), ("sin", sin)):
+            _need(t is not None and t.dtype == torch.float32 and t.dim() == 2 and t.shape[1] == rotary_dim // 2
+                  and t.is_contiguous(), f"{name} must be contiguous float32 [positions, rotary_dim / 2]")
+    _check_kv_pages(k_pages, v_pages, num_kv_heads, page_size, key_dim, value_dim, q.dtype)
+    _i32(positions, "positions", tokens)
+    _i32(slot_of_token, "slot_of_token", tokens)
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
+          "block_table must be contiguous int32 [slots, pages]")
+    lib.call("arle_rotary_qkv_store", q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0),
+             _code(q), _ptr(q_weight), _ptr(k_weight), w_code, float(eps), 1 if unit_after else 0, _ptr(cos), _ptr(sin),
+             int(rotary_dim), 1 if interleaved else 0, positions.data_ptr(), slot_of_token.data_ptr(),
+             block_table.data_ptr(), block_table.shape[1], k_pages.data_ptr(), v_pages.data_ptr(), tokens, num_q_heads,
+             num_kv_heads, key_dim, value_dim, int(page_size), _stream())
+
+
+# ------------------------------------------------------------------------- gated delta rule
+
+GATED_DELTA_MAX_KEY_DIM = 256
+
+
+def gated_delta_scan(q, k, v, gates, a_log, dt_bias, s_state, seg_row0, seg_slot, *, heads: int, kv_heads: int,
+                     key_dim: int, value_dim: int, unit_eps: float = 1e-6):
+    """The gated delta rule over the rows of every segment, from and into the requests' states (see
+    csrc/gated_delta.hip).  q, k [T, kv_heads * D] and v [T, heads * Dv] as the convolutions left them; gates float32
+    [T, >= 2 * heads]: the pre-activations of beta, then those of the decay; a_log, dt_bias float32 [heads]; s_state
+    float32 [slots, heads, D, Dv].  Returns o float32 [T, heads * Dv]."""
+    _gpu(q, k, v, gates, a_log, dt_bias, s_state, seg_row0, seg_slot)
+    H, G, D, Dv = heads, kv_heads, key_dim, value_dim
+    tokens = q.shape[0]
+    for name, t, width in (("q", q, G * D), ("k", k, G * D), ("v", v, H * Dv)):
+        _rows(t, name)
+        _need(t.shape == (tokens, width) and t.dtype == q.dtype and t.dtype in _CODES, f"{name} must be [T, {width}] of one type")
+    _need(0 < D <= GATED_DELTA_MAX_KEY_DIM and G > 0 and H % G == 0 and H <= _GRID_Y_MAX,
+          f"key sizes up to {GATED_DELTA_MAX_KEY_DIM}, heads a multiple of the q/k heads")
+    _rows(gates, "gates")
+    _need(gates.dtype == torch.float32 and gates.shape[0] == tokens and gates.shape[1] >= 2 * H, "gates must be float32 [T, >= 2 * heads]")
+    _need(a_log.shape == (H,) and dt_bias.shape == (H,) and a_log.dtype == dt_bias.dtype == torch.float32
+          and a_log.is_contiguous() and dt_bias.is_contiguous(), "A_log and dt_bias must be float32 [heads]")
+    _need(s_state.dim() == 4 and tuple(s_state.shape[1:]) == (H, D, Dv) and s_state.dtype == torch.float32
+          and s_state.is_contiguous(), "the state is float32 [slots, heads, D, Dv]")
+    segments = seg_slot.numel()
+    _i32(seg_slot, "seg_slot")
+    _i32(seg_row0, "seg_row0", segments + 1)
+    out = torch.empty((tokens, H * Dv), dtype=torch.float32, device=q.device)
+    lib.call("arle_gated_delta_scan", q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0),
+             _code(q), gates.data_ptr(), gates.stride(0), a_log.data_ptr(), dt_bias.data_ptr(), float(unit_eps),
+             s_state.data_ptr(), seg_row0.data_ptr(), seg_slot.data_ptr(), segments, out.data_ptr(), H, G, D, Dv, _stream())
+    return out
+
+
+def gated_delta_output(o, gate, weight, eps: float, *, heads: int, value_dim: int):
+    """Each head's o [T, heads * Dv] (float32) divided by its root mean square, times weight [Dv], times silu(gate);
+    in the type of `gate`."""
+    _gpu(o, gate, weight)
+    tokens = o.shape[0]
+    width = heads * value_dim
+    _need(o.dtype == torch.float32 and o.shape == (tokens, width) and o.is_contiguous(), "o must be float32 [T, H * Dv]")
+    _rows(gate, "gate")
+    _need(gate.shape == (tokens, width) and gate.dtype in _CODES, "gate must be [T, H * Dv]")
+    _need(weight.shape == (value_dim,) and weight.is_contiguous() and weight.dtype in _CODES, "the norm weight must be [Dv]")
+    _need(heads <= _GRID_Y_MAX, "too many heads")
+    out = torch.empty((tokens, width), dtype=gate.dtype, device=o.device)
+    lib.call("arle_gated_delta_output", o.data_ptr(), gate.data_ptr(), gate.stride(0), _code(gate), weight.data_ptr(),
+             _code(weight), float(eps), out.data_ptr(), tokens, heads, value_dim, _stream())
     return out

@@ -12,8 +12,9 @@ import sys
 
 from ..kernels import ops
 from ..parts import base  # noqa: F401  (registries)
-from ..parts import (attention, block, embedding, feed_forward, latent_attention, mlstm, moe, norm,  # noqa: F401  registers the stock parts
-                     position, short_conv, softcap_attention, wide_norm_attention)
+from ..parts import (attention, block, embedding, feed_forward, gated_delta, hyper, latent_attention,  # noqa: F401  registers the stock parts
+                     mixer_pair, mlstm, moe, norm, position, rotary_attention, short_conv, softcap_attention,
+                     wide_norm_attention)
 from ..parts.base import Runtime, build_part, expected_tensors, lookup
 from ..parts.spec import ModelSpec
 
@@ -74,6 +75,9 @@ def debug_dump(residual, delta, label: str) -> None:
     schedule entry (first and last values, minimum, maximum, root mean square, NaN or infinity anywhere), as the
     reference prints with INFER_DEBUG_DUMP (infer/src/model/common.rs:85-124).  Synchronises; steps are then not
     captured."""
+    if residual.dim() == 3 or hasattr(delta, "settled"):      # residual streams: their sum, a pending write done
+        residual = delta.settled(residual) if hasattr(delta, "settled") else residual.sum(1)
+        delta = None
     row = residual[-1].float()
     terms = delta if isinstance(delta, list) else ([] if delta is None else [(delta, None)])
     for term, bias in terms:

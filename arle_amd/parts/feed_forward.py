@@ -17,7 +17,8 @@ from .linear import Linear
 @register("feed_forward", "swiglu")
 class SwiGLU(Part):
     """params: hidden_size, intermediate_size, float32_out (bool, default False: the down projection hands on its
-    32-bit sums instead of rounding them to the activation type)."""
+    32-bit sums instead of rounding them to the activation type), activation ("silu", the default, or "gelu_tanh":
+    what the gate passes through before it multiplies up)."""
 
     graph_safe = True  # launches depend on shapes only, never on the values of a step
 
@@ -30,6 +31,10 @@ class SwiGLU(Part):
         super().__init__(params, tensors, rt, children)
         self.inter = int(params["intermediate_size"])
         self.float32_out = bool(params.get("float32_out", False))
+        name = params.get("activation") or "silu"
+        if name not in ops.ACTIVATIONS:
+            raise ValueError(f"unknown activation {name!r} (known: {', '.join(ops.ACTIVATIONS)})")
+        self.act = ops.ACTIVATIONS[name]
         gate, up = tensors["gate"], tensors["up"]
         if gate.dtype != up.dtype:
             raise ValueError("gate and up projections must be stored in one type")
@@ -54,10 +59,10 @@ class SwiGLU(Part):
     def forward(self, x):
         """x [T, H] -> [T, H], or a float32 stack [S, T, H] to be added in order (see Linear)."""
         if self.block:
-            act = ops.gate_up_act(x, self.gate_up.weight, self.gate_up.tiles)   # one product with the activation, or two kernels
+            act = ops.gate_up_act(x, self.gate_up.weight, self.gate_up.tiles, self.act)   # one product with the activation, or two kernels
         else:
             gu = self.gate_up(x)
-            act = ops.silu_mul(gu[:, : self.inter], gu[:, self.inter:])
+            act = ops.act_mul(gu[:, : self.inter], gu[:, self.inter:], self.act)
         return self.down(act, out_dtype=torch.float32 if self.float32_out else None, partials_ok=True)
 
 

@@ -27,10 +27,10 @@ class ShortConv:
         """The state of a convolution of `taps` taps: its last taps - 1 inputs, in the activation type."""
         return StateNeed((taps - 1, channels), None) if taps > 1 else None
 
-    def __call__(self, u, batch, state_view, add_input: bool = False):
-        """The convolution of the step's rows; the requests' states move on by the rows they brought."""
+    def __call__(self, u, batch, state_view, add_input: bool = False, silu: bool = False):
+        """The convolution of the step's rows (with `silu`, its silu); the requests' states move on by the rows they brought."""
         state = state_view.state if (state_view is not None and self.taps > 1) else None
-        y = ops.causal_conv(u, self.weight, state, batch.slot_of_token, bias=self.bias, add_input=add_input)
+        y = ops.causal_conv(u, self.weight, state, batch.slot_of_token, bias=self.bias, add_input=add_input, silu=silu)
         if state is not None:
             ops.conv_state_update(u, state, batch.seg_row0, batch.seg_slot, bias=self.bias)
         return y

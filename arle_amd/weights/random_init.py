@@ -47,8 +47,25 @@ def _init_near_zero(shape, gen, std, norm_std, device):
     return t
 
 
+def _init_stream_in(shape, gen, std, norm_std, device):
+    """What a sublayer reads of residual streams: their mean, 1 / streams + N(0, norm_std)."""
+    t = torch.full(shape, 1.0 / max(shape[0], 1), dtype=torch.float32, device=device)
+    if norm_std:
+        t += torch.randn(shape, generator=gen, dtype=torch.float32, device=device) * norm_std
+    return t
+
+
+def _init_stream_mix(shape, gen, std, norm_std, device):
+    """How residual streams pass a sublayer: each into itself, the identity + N(0, norm_std)."""
+    t = torch.eye(shape[0], shape[1], dtype=torch.float32, device=device)
+    if norm_std:
+        t += torch.randn(shape, generator=gen, dtype=torch.float32, device=device) * norm_std
+    return t
+
+
 # WeightDecl.init -> how a random tensor of that kind is filled: f(shape, generator, std, norm_std, device) -> float32
-INITS = {"normal": _init_normal, "ones": _init_ones, "zeros": _init_zeros, "near_zero": _init_near_zero}
+INITS = {"normal": _init_normal, "ones": _init_ones, "zeros": _init_zeros, "near_zero": _init_near_zero,
+         "stream_in": _init_stream_in, "stream_mix": _init_stream_mix}
 
 
 def register_init(name: str, fill) -> None:
