@@ -12,7 +12,8 @@ from .base import register
 
 @register("block", "pre_norm")
 class PreNormBlock:
-    """norm roles: "mixer_in", "ffn_in"."""
+    """norm roles: "mixer_in", "ffn_in" (the second only with a feed-forward; without one the mixer's output is what
+    the next block adds)."""
 
     norm_roles = ("mixer_in", "ffn_in")
 
@@ -21,11 +22,13 @@ class PreNormBlock:
         self.feed_forward = feed_forward
         self.norms = norms
         self.norm_mixer = norms["mixer_in"]
-        self.norm_ffn = norms["ffn_in"]
+        self.norm_ffn = norms["ffn_in"] if feed_forward is not None else None
 
     def forward(self, residual, delta, batch, cache_view):
         a = self.norm_mixer.add_norm(residual, delta)
         m = self.mixer.forward(a, batch, cache_view)
+        if self.norm_ffn is None:
+            return residual, m
         b = self.norm_ffn.add_norm(residual, m)
         return residual, self.feed_forward.forward(b)
 

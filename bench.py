@@ -5,6 +5,7 @@
     python bench.py --generate                                       (the decode workload through LLM.generate)
     python bench.py --workload gufasun [--shape 4b|8b] [--layers L]  (the Gufasun design beside Qwen3 at equal sizes)
     python bench.py --workload sovutar [--shape 4b|8b] [--layers L]  (the Sovutar design beside Qwen3 at equal sizes)
+    python bench.py --workload tazitar [--shape 4b|8b] [--layers L]  (the Tazitar design beside Qwen3 at equal sizes)
 
 A step is one decode step of `batch` requests, each holding a `prompt`-token random prompt
 (prefilled by the engine itself before the clock starts) and growing by one token per step.
@@ -834,6 +835,74 @@ def sovutar_work(raw: dict, q: dict, tokens: int, batch: int, context: int) -> d
     }
 
 
+# ---- the Tazitar design beside Qwen3 at equal sizes -------------------------------------------------------
+# The widths and head counts of Qwen3-4B / 8B over four residual streams; the layers cycle through the three mixers
+# (capped attention with q/k norm; an attention with a sink beside a gated delta rule; an attention with interleaved
+# YaRN rotation and a learned sink), and from eight layer runs on, layers 1..3 run twice with the same weights.
+def tazitar_config(shape: str, layers: int) -> dict:
+    q = SOVUTAR_SHAPES[shape][0]
+    H, G, D = q["num_attention_heads"], q["num_key_value_heads"], q["head_dim"]
+    attn = {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5, "softcap": 30.0,
+            "rot": {"base": 1000000.0, "dims": D}}
+    left = {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": 0.3, "rot": {"base": 1000000.0, "dims": D // 2}}
+    right = {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "conv": 4}
+    attn2 = {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": 0.3,
+             "rot": {"base": 1000000.0, "dims": D, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+    kinds = [("attention", attn), ("parallel", {"left": left, "right": right}), ("attention_2", attn2)]
+    mlp = {"kind": "dense", "ff": q["intermediate_size"]}
+    loop = {"start": 1, "stop": 4, "times": 2} if layers >= 8 else None
+    unique = layers - 3 if loop else layers
+    out = [{"type": kinds[i % 3][0], "mixer": json.loads(json.dumps(kinds[i % 3][1])), "mlp": dict(mlp)} for i in range(unique)]
+    raw = {"architecture": "Tazitar", "vocab": q["vocab_size"], "width": q["hidden_size"], "norm": {"eps": 1e-6},
+           "streams": 4, "layers": out}
+    if loop:
+        raw["loop"] = loop
+    return raw
+
+
+def tazitar_work(raw: dict, q: dict, tokens: int, batch: int, context: int) -> dict:
+    """Ideal work of the kernels that are new with this design, per step: kernel family -> (bytes, flops)."""
+    from arle_amd.config import TazitarConfig
+
+    order = TazitarConfig.from_dict(raw).layer_order()
+    runs = [raw["layers"][i] for i in order]
+    W, S, L = raw["width"], raw["streams"], len(runs)
+    F = runs[0]["mlp"]["ff"]
+    n_par = sum(l["type"] == "parallel" for l in runs)
+    a = next(l["mixer"] for l in runs if l["type"] == "attention")
+    r = next(l["mixer"]["right"] for l in runs if l["type"] == "parallel") if n_par else None
+    H, G, D, Dv = a["heads"], a["kv_heads"], a["dim"], a["vdim"]
+    decode = tokens == batch
+    keys = context if decode else tokens / 2
+    work = {
+        "hyper_step_kernel": ((2 * L + 1) * tokens * W * (8 * S + 4 + 2), 0),
+        "rotary_qkv_store_kernel": (L * tokens * (H * D + G * D + G * Dv) * 4, 0),
+        "attn_softcap_mfma_kernel": (L * batch * keys * G * (D + Dv) * 2 if decode else 0, L * tokens * keys * H * 2 * (D + Dv)),
+        "silu_mul_bf16x8_kernel": (L * tokens * F * 6, 0),
+    }
+    if r is not None:
+        state = r["heads"] * r["dim"] * r["vdim"]
+        conv = 2 * r["kv_heads"] * r["dim"] + r["heads"] * r["vdim"]
+        work.update({
+            "pair_norm_kernel": (n_par * tokens * W * 12, 0),
+            "causal_conv": (n_par * tokens * conv * 4, 0),
+            "gated_delta_scan_kernel": (n_par * batch * state * 8, n_par * tokens * state * 6),
+            "gated_delta_output_kernel": (n_par * tokens * r["heads"] * r["vdim"] * 8, 0),
+        })
+    return work
+
+
+def tazitar_bench(args) -> int:
+    """Prefill and decode throughput of the Tazitar design and of Qwen3 at the same widths and depth."""
+    from arle_amd.config import Qwen3Config, TazitarConfig
+
+    layers = args.layers if args.layers != FULL_LAYERS else 8
+    q = dict(SOVUTAR_SHAPES[args.shape][0], num_hidden_layers=layers)
+    raw = tazitar_config(args.shape, layers)
+    models = {"tazitar": ("Tazitar", TazitarConfig.from_dict(raw)), "qwen3": ("Qwen3ForCausalLM", Qwen3Config.from_dict(q))}
+    return design_bench(args, "tazitar", models, q, layers, lambda tokens, batch, context: tazitar_work(raw, q, tokens, batch, context))
+
+
 def sovutar_bench(args) -> int:
     """Prefill and decode throughput of the Sovutar design and of Qwen3 at the same widths and depth."""
     from arle_amd.config import Qwen3Config, SovutarConfig
@@ -981,10 +1050,10 @@ def main() -> int:
                          "and write the table that ARLE_AMD_PRODUCT_TABLE / ops.load_product_table reads; WIDTHS: 4b, 8b, "
                          "32b or hidden,q_width,kv_width,intermediate[,vocabulary]")
     ap.add_argument("--out", default=None, help="--tune-products: the table's file (default: product_table_<widths>.json)")
-    ap.add_argument("--workload", default="qwen3-4b", choices=["qwen3-4b", "qwen3-8b-mixed", "qwen3-32b-decode", "gufasun", "sovutar"],
+    ap.add_argument("--workload", default="qwen3-4b", choices=["qwen3-4b", "qwen3-8b-mixed", "qwen3-32b-decode", "gufasun", "sovutar", "tazitar"],
                     help="qwen3-4b is the default run; the next two are further workloads at larger shapes; gufasun: "
                          "the Gufasun design beside Qwen3 at equal widths and depth (--shape, --layers, --batch, --prompt-len)")
-    ap.add_argument("--shape", default="4b", choices=["4b", "8b"], help="--workload gufasun / sovutar: whose widths")
+    ap.add_argument("--shape", default="4b", choices=["4b", "8b"], help="--workload gufasun / sovutar / tazitar: whose widths")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for --gpus {args.gpus})")
@@ -1008,6 +1077,8 @@ def main() -> int:
         return gufasun_bench(args)
     if args.workload == "sovutar":
         return sovutar_bench(args)
+    if args.workload == "tazitar":
+        return tazitar_bench(args)
     if args.workload == "qwen3-4b" and args.batch is None:
         args.batch = 8
     if args.workload != "qwen3-4b":

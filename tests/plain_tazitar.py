@@ -24,6 +24,17 @@ def rms_unit(x, eps):
     return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
 
 
+# A test may set this to a function of a matrix product's output (to model the rounding of activations); None in
+# ordinary use.
+after_product = None
+
+
+def lin(h, weight):
+    """weight [out, in] applied to the rows of h."""
+    y = h @ weight.T
+    return y if after_product is None else after_product(y)
+
+
 def gelu_tanh(z):
     return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
 
@@ -48,7 +59,9 @@ def rotary_frequencies(rot, dtype=torch.float32):
 
 def rotate(x, positions, rot, interleaved):
     """x [T, heads, D]: the first rot.dims entries of every head are rotated by the angle p f_i; pairs are
-    (i, i + dims/2) or, interleaved, (2i, 2i + 1)."""
+    (i, i + dims/2) or, interleaved, (2i, 2i + 1).  rot None: nothing rotates."""
+    if rot is None:
+        return x
     dims = int(rot["dims"])
     f, mag = rotary_frequencies(rot, x.dtype)
     angle = positions.to(x.dtype)[:, None] * f[None, :]
@@ -95,22 +108,22 @@ def attention(h, w, p, m, eps, positions, kind):
     kind "sink0": rotate-half rotation, then unit-rms q and k, a sink of score 0.
     kind "attention_2": interleaved rotation (YaRN), then unit-rms q and k, a learned sink."""
     T = h.shape[0]
-    H, G, D, Dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    q = (h @ w[p + "q"].T).view(T, H, D)
-    k = (h @ w[p + "k"].T).view(T, G, D)
-    v = (h @ w[p + "v"].T).view(T, G, Dv)
+    H, G, D, Dv = m["heads"], m.get("kv_heads") or m["heads"], m["dim"], m["vdim"]
+    q = lin(h, w[p + "q"]).view(T, H, D)
+    k = lin(h, w[p + "k"]).view(T, G, D)
+    v = lin(h, w[p + "v"]).view(T, G, Dv)
     sink = None
     if kind == "attention":
         q = rms_unit(q, eps) * w[p + "q.norm"]
         k = rms_unit(k, eps) * w[p + "k.norm"]
-        q, k = rotate(q, positions, m["rot"], False), rotate(k, positions, m["rot"], False)
+        q, k = rotate(q, positions, m.get("rot"), False), rotate(k, positions, m.get("rot"), False)
     else:
         inter = kind == "attention_2"
-        q, k = rotate(q, positions, m["rot"], inter), rotate(k, positions, m["rot"], inter)
+        q, k = rotate(q, positions, m.get("rot"), inter), rotate(k, positions, m.get("rot"), inter)
         q, k = rms_unit(q, eps), rms_unit(k, eps)
         sink = w[p + "sink"] if inter else torch.zeros(H, dtype=h.dtype)
     o = causal_softmax_attention(q, k, v, m["scale"], m.get("softcap"), sink)
-    return o @ w[p + "o"].T
+    return lin(o, w[p + "o"])
 
 
 def short_conv(x, weight):
@@ -122,15 +135,15 @@ def short_conv(x, weight):
 
 def gated_delta_rule(h, w, p, m, eps):
     T = h.shape[0]
-    H, G, D, Dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    q = F.silu(short_conv(h @ w[p + "q"].T, w[p + "q.conv"])).view(T, G, D)
-    k = F.silu(short_conv(h @ w[p + "k"].T, w[p + "k.conv"])).view(T, G, D)
-    v = F.silu(short_conv(h @ w[p + "v"].T, w[p + "v.conv"])).view(T, H, Dv)
+    H, G, D, Dv = m["heads"], m.get("kv_heads") or m["heads"], m["dim"], m["vdim"]
+    q = F.silu(short_conv(lin(h, w[p + "q"]), w[p + "q.conv"])).view(T, G, D)
+    k = F.silu(short_conv(lin(h, w[p + "k"]), w[p + "k.conv"])).view(T, G, D)
+    v = F.silu(short_conv(lin(h, w[p + "v"]), w[p + "v.conv"])).view(T, H, Dv)
     unit = lambda x: x / torch.sqrt((x * x).sum(-1, keepdim=True) + 1e-6)
     q, k = unit(q) * D ** -0.5, unit(k)
     q, k = q.repeat_interleave(H // G, dim=1), k.repeat_interleave(H // G, dim=1)
-    beta = torch.sigmoid(h @ w[p + "b"].T)                                               # [T, H]
-    decay = torch.exp(-torch.exp(w[p + "A_log"]) * F.softplus(h @ w[p + "a"].T + w[p + "dt_bias"]))
+    beta = torch.sigmoid(lin(h, w[p + "b"]))                                               # [T, H]
+    decay = torch.exp(-torch.exp(w[p + "A_log"]) * F.softplus(lin(h, w[p + "a"]) + w[p + "dt_bias"]))
     S = h.new_zeros(H, D, Dv)
     out = h.new_zeros(T, H, Dv)
     for t in range(T):
@@ -138,9 +151,9 @@ def gated_delta_rule(h, w, p, m, eps):
         u = beta[t][:, None] * (v[t] - torch.einsum("hdv,hd->hv", S, k[t]))
         S = S + k[t][:, :, None] * u[:, None, :]
         out[t] = torch.einsum("hdv,hd->hv", S, q[t])
-    gate = F.silu(h @ w[p + "g"].T).view(T, H, Dv)
+    gate = F.silu(lin(h, w[p + "g"])).view(T, H, Dv)
     y = rms_unit(out, eps) * w[p + "norm"] * gate
-    return y.reshape(T, -1) @ w[p + "o"].T
+    return lin(y.reshape(T, -1), w[p + "o"])
 
 
 def parallel_mixer(h, w, p, m, eps, positions):
@@ -150,7 +163,7 @@ def parallel_mixer(h, w, p, m, eps, positions):
 
 
 def feed_forward(h, w, p):
-    return (gelu_tanh(h @ w[p + "gate"].T) * (h @ w[p + "up"].T)) @ w[p + "down"].T
+    return lin(gelu_tanh(lin(h, w[p + "gate"])) * lin(h, w[p + "up"]), w[p + "down"])
 
 
 def layer_order(config):
