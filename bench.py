@@ -876,7 +876,7 @@ def tazitar_work(raw: dict, q: dict, tokens: int, batch: int, context: int) -> d
     keys = context if decode else tokens / 2
     work = {
         "hyper_step_kernel": ((2 * L + 1) * tokens * W * (8 * S + 4 + 2), 0),
-        "rotary_qkv_store_kernel": (L * tokens * (H * D + G * D + G * Dv) * 4, 0),
+        "rotary_qkv_store_x8_kernel": (L * tokens * (H * D + G * D + G * Dv) * 4, 0),
         "attn_softcap_mfma_kernel": (L * batch * keys * G * (D + Dv) * 2 if decode else 0, L * tokens * keys * H * 2 * (D + Dv)),
         "silu_mul_bf16x8_kernel": (L * tokens * F * 6, 0),
     }
