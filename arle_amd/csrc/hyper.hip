@@ -4,7 +4,9 @@
 // `hyper_step`: instead of one residual a token has S streams x_1..x_S, float32 [T, S, W].  A sublayer with the
 // connection (a[S], b[S], M[S, S]) reads  N(sum_s a_s x_s)  and its output y is written as
 //     x_t <- sum_s M[s, t] x_s + b_t y        (all streams at once from the old ones).
-// One launch does the write of the sublayer before and the read of the next one, a workgroup a token:
+// One launch does the write of the sublayer before and the read of the next one, a workgroup a token (256 threads
+// where the step has rows enough to fill the chip, else up to 1,024, so that a decoded row's columns are loaded in one
+// round instead of several that wait for each other):
 //     x' = write(x, y; M, b)   (y null: x' = x);   u = sum_t a_t x'_t   (a null: the plain sum);
 //     out = u / sqrt(mean(u^2) + eps) * w   in the activation type.
 // The input streams may be one row for all streams (stream stride 0: every stream starts as a copy of the
@@ -36,8 +38,8 @@ __device__ __forceinline__ void load_y(const TY* y, int parts, int64_t part_stri
   }
 }
 
-template <typename TY, typename TA, int SMAX, int VEC>
-__global__ __launch_bounds__(kHyThreads) void hyper_step_kernel(
+template <typename TY, typename TA, int SMAX, int VEC, int THREADS>
+__global__ __launch_bounds__(THREADS) void hyper_step_kernel(
     const float* x_in, long long in_row_stride, long long in_stream_stride, float* x_out,   // may be the same memory
     const TY* __restrict__ y, long long y_stride, int y_parts, long long y_part_stride, const float* __restrict__ mix,
     const float* __restrict__ out_w, const float* __restrict__ in_w, const float* __restrict__ norm_w, float eps,
@@ -48,7 +50,7 @@ __global__ __launch_bounds__(kHyThreads) void hyper_step_kernel(
   const float* src = x_in + t * in_row_stride;
   float* dst = (x_out && !rows) ? x_out + t * static_cast<int64_t>(S) * W : nullptr;
   float ss = 0.f;
-  for (int c = threadIdx.x * VEC; c < W; c += kHyThreads * VEC) {
+  for (int c = threadIdx.x * VEC; c < W; c += THREADS * VEC) {
     float x[SMAX][VEC];
 #pragma unroll
     for (int s = 0; s < SMAX; ++s) {
@@ -119,9 +121,9 @@ __global__ __launch_bounds__(kHyThreads) void hyper_step_kernel(
       ss = fmaf(u[e], u[e], ss);
     }
   }
-  const float inv = 1.0f / sqrtf(block_sum<kHyThreads / kWave>(ss, red) / static_cast<float>(W) + eps);
+  const float inv = 1.0f / sqrtf(block_sum<THREADS / kWave>(ss, red) / static_cast<float>(W) + eps);
   TA* o = out + static_cast<int64_t>(blockIdx.x) * out_stride;
-  for (int c = threadIdx.x * VEC; c < W; c += kHyThreads * VEC) {
+  for (int c = threadIdx.x * VEC; c < W; c += THREADS * VEC) {
     if constexpr (VEC == 4) {
       const float4 w = *reinterpret_cast<const float4*>(norm_w + c);
       st4<TA>(o + c, float4{u_lds[c] * inv * w.x, u_lds[c + 1] * inv * w.y, u_lds[c + 2] * inv * w.z, u_lds[c + 3] * inv * w.w});
@@ -166,12 +168,20 @@ int launch_hyper(const float* x_in, long long in_row_stride, long long in_stream
                  long long y_stride, int y_parts, long long y_part_stride, const float* mix, const float* out_w,
                  const float* in_w, const float* norm_w, float eps, const int* rows, void* out, long long out_stride,
                  int grid, int S, int W, hipStream_t s) {
-  const size_t lds = (static_cast<size_t>(W) + kHyThreads / kWave) * sizeof(float);
-#define ARLE_HYPER(SMAX)                                                                                             \
-  hyper_step_kernel<TY, TA, SMAX, VEC><<<grid, kHyThreads, lds, s>>>(                                                \
+  const size_t lds = (static_cast<size_t>(W) + 1024 / kWave) * sizeof(float);
+  // few rows: as many threads a row as its columns ask for, up to 1,024 (S <= 4 only: more streams are more registers)
+  // (bfloat16 steps only: in float32 a row's sums run in one order whatever else the step holds)
+  const bool wide = sizeof(TA) == 2 && grid < 512 && S <= 4 && W > kHyThreads * VEC;
+#define ARLE_HYPER_T(SMAX, THREADS)                                                                                  \
+  hyper_step_kernel<TY, TA, SMAX, VEC, THREADS><<<grid, THREADS, lds, s>>>(                                          \
       x_in, in_row_stride, in_stream_stride, x_out, static_cast<const TY*>(y), y_stride, y_parts, y_part_stride, mix, \
       out_w, in_w, norm_w, eps, rows, static_cast<TA*>(out), out_stride, S, W)
+#define ARLE_HYPER(SMAX)                                                                                             \
+  do {                                                                                                               \
+    if (wide && SMAX <= 4) ARLE_HYPER_T(SMAX <= 4 ? SMAX : 4, 1024); else ARLE_HYPER_T(SMAX, kHyThreads);            \
+  } while (0)
   if (S <= 2) ARLE_HYPER(2); else if (S <= 4) ARLE_HYPER(4); else if (S <= 8) ARLE_HYPER(8); else ARLE_HYPER(16);
+#undef ARLE_HYPER_T
 #undef ARLE_HYPER
   return launch_status();
 }
