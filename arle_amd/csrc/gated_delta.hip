@@ -10,7 +10,13 @@
 // 32; the block's unit norms, gates and the dot products k . q are made there, a row by eight threads, always
 // the same entries in the same order.  The chain of a row is one pass over the lane's share of the old S for both
 // S^T k and S^T q (o = g S_old^T q + u (k . q), which is S_new^T q), one exchange over the sixteen shares, and the
-// update.  `gated_delta_output` divides each head's o by its root mean square, multiplies by the norm's weight and
+// update.  Two layouts of a wave, which add the sixteen shares in the same tree and so give the same bits.  ROWS
+// (steps with portions): the sixteen shares of a column are the sixteen lanes of a row of the wave, and the exchange
+// is four data-parallel-primitive moves inside the vector unit (neighbours, pairs, the mirrored half, the mirrored
+// row), never through LDS, whose unit the rows' reads of q and k keep busy.  Otherwise (steps of decoded rows, whose
+// time is the state's way in and out): the four columns of a wave are four neighbouring lanes, so that a load of the
+// state is sixteen bytes for every four lanes, and the shares exchange through lane reads four, eight, sixteen and
+// 32 lanes away.  `gated_delta_output` divides each head's o by its root mean square, multiplies by the norm's weight and
 // by silu of the gate's projection.
 #include "common.h"
 
@@ -26,7 +32,22 @@ constexpr int kGdRowThreads = kGdThreads / kGdRows;   // threads that prepare a 
 
 __device__ __forceinline__ float softplus(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
 
-template <typename T, int DS>
+// The sum of v over the sixteen lanes of a row, in every lane of the row, the same bits in each: lane i adds lane
+// i ^ 1, then i ^ 2 (afterwards the four lanes of a quad agree), then the lane mirrored in its half (the other quad's
+// sum), then the lane mirrored in its row (the other half's sum).
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float row16_sum(float v) {
+  v += dpp_move<0xB1>(v);    // quad_perm [1, 0, 3, 2]
+  v += dpp_move<0x4E>(v);    // quad_perm [2, 3, 0, 1]
+  v += dpp_move<0x141>(v);   // row_half_mirror
+  v += dpp_move<0x140>(v);   // row_mirror
+  return v;
+}
+
+template <typename T, int DS, bool ROWS>
 __global__ __launch_bounds__(kGdThreads) void gated_delta_scan_kernel(
     const T* __restrict__ q, long long q_stride, const T* __restrict__ k, long long k_stride, const T* __restrict__ v,
     long long v_stride, const float* __restrict__ gates /* [T, >= 2H]: b then a */, long long gates_stride,
@@ -41,9 +62,10 @@ __global__ __launch_bounds__(kGdThreads) void gated_delta_scan_kernel(
   const int seg = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int lane = tid % kWave, wave = tid / kWave;
   const int kvh = h / (H / G);
-  const int col_in = wave * kGdWaveCols + lane % kGdWaveCols;
+  static_assert(kGdParts == 16, "a column's shares are the lanes of one row of sixteen");
+  const int col_in = wave * kGdWaveCols + (ROWS ? lane / kGdParts : lane % kGdWaveCols);
   const int col = blockIdx.z * kGdCols + col_in;
-  const int part = lane / kGdWaveCols;
+  const int part = ROWS ? lane % kGdParts : lane / kGdWaveCols;
   const bool live = col < Dv;
   const int row0 = seg_row0[seg], rows = seg_row0[seg + 1] - row0;
   float* s_ptr = s_state + (static_cast<int64_t>(seg_slot[seg]) * H + h) * D * Dv;
@@ -61,35 +83,37 @@ __global__ __launch_bounds__(kGdThreads) void gated_delta_scan_kernel(
     {   // a row by kGdRowThreads threads: its q and k to LDS, their unit norms, k . q, the gates
       const int r = tid / kGdRowThreads, sub = tid % kGdRowThreads;
       const int64_t t = row0 + base + min(r, n - 1);
-      const T* qr = q + t * q_stride + kvh * D;
-      const T* kr = k + t * k_stride + kvh * D;
-      float sq = 0.f, sk = 0.f, kq = 0.f;
-      for (int d = sub; d < DP; d += kGdRowThreads) {
-        const float qv = d < D ? to_float(qr[d]) : 0.f, kv = d < D ? to_float(kr[d]) : 0.f;
-        q_lds[r][d] = qv;
-        k_lds[r][d] = kv;
-        sq = fmaf(qv, qv, sq);
-        sk = fmaf(kv, kv, sk);
-        kq = fmaf(kv, qv, kq);
-      }
+      if (r < n) {   // (the threads of a row leave or stay together; a decoded row's block is one row)
+        const T* qr = q + t * q_stride + kvh * D;
+        const T* kr = k + t * k_stride + kvh * D;
+        float sq = 0.f, sk = 0.f, kq = 0.f;
+        for (int d = sub; d < DP; d += kGdRowThreads) {
+          const float qv = d < D ? to_float(qr[d]) : 0.f, kv = d < D ? to_float(kr[d]) : 0.f;
+          q_lds[r][d] = qv;
+          k_lds[r][d] = kv;
+          sq = fmaf(qv, qv, sq);
+          sk = fmaf(kv, kv, sk);
+          kq = fmaf(kv, qv, kq);
+        }
 #pragma unroll
-      for (int off = kGdRowThreads / 2; off > 0; off >>= 1) {
-        sq += __shfl_xor(sq, off, kWave);
-        sk += __shfl_xor(sk, off, kWave);
-        kq += __shfl_xor(kq, off, kWave);
+        for (int off = kGdRowThreads / 2; off > 0; off >>= 1) {
+          sq += __shfl_xor(sq, off, kWave);
+          sk += __shfl_xor(sk, off, kWave);
+          kq += __shfl_xor(kq, off, kWave);
+        }
+        const float fq = q_scale / sqrtf(sq + unit_eps), fk = 1.0f / sqrtf(sk + unit_eps);
+        for (int d = sub; d < DP; d += kGdRowThreads) {   // the entries this thread has written itself
+          q_lds[r][d] *= fq;
+          k_lds[r][d] *= fk;
+        }
+        if (sub == 0) {
+          const float b = gates[t * gates_stride + h], a = gates[t * gates_stride + H + h];
+          c_lds[r][0] = expf(-rate * softplus(a + bias));
+          c_lds[r][1] = 1.0f / (1.0f + expf(-b));
+          c_lds[r][2] = kq * fq * fk;
+        }
       }
-      const float fq = q_scale / sqrtf(sq + unit_eps), fk = 1.0f / sqrtf(sk + unit_eps);
-      for (int d = sub; d < DP; d += kGdRowThreads) {   // the entries this thread has written itself
-        q_lds[r][d] *= fq;
-        k_lds[r][d] *= fk;
-      }
-      if (sub == 0) {
-        const float b = gates[t * gates_stride + h], a = gates[t * gates_stride + H + h];
-        c_lds[r][0] = expf(-rate * softplus(a + bias));
-        c_lds[r][1] = 1.0f / (1.0f + expf(-b));
-        c_lds[r][2] = kq * fq * fk;
-      }
-      for (int e = tid; e < kGdRows * kGdCols; e += kGdThreads) {
+      for (int e = tid; e < n * kGdCols; e += kGdThreads) {
         const int rr = e / kGdCols, cc = e % kGdCols;
         const int64_t tt = row0 + base + min(rr, n - 1);
         const int c_abs = min(static_cast<int>(blockIdx.z) * kGdCols + cc, Dv - 1);
@@ -119,10 +143,15 @@ __global__ __launch_bounds__(kGdThreads) void gated_delta_scan_kernel(
       }
 #pragma unroll
       for (int i = 0; i < DS; ++i) dk = fmaf(S[i], kk[i], dk);
+      if constexpr (ROWS) {   // over the shares of D: with share p ^ 1, then p ^ 2, p ^ 4, p ^ 8
+        dk = row16_sum(dk);
+        dq = row16_sum(dq);
+      } else {
 #pragma unroll
-      for (int off = kGdWaveCols; off < kWave; off <<= 1) {   // over the shares of D, in a fixed order
-        dk += __shfl_xor(dk, off, kWave);
-        dq += __shfl_xor(dq, off, kWave);
+        for (int off = kGdWaveCols; off < kWave; off <<= 1) {
+          dk += __shfl_xor(dk, off, kWave);
+          dq += __shfl_xor(dq, off, kWave);
+        }
       }
       const float u = beta * (v_lds[r][col_in] - g * dk);
 #pragma unroll
@@ -162,14 +191,16 @@ using namespace arle;
 extern "C" int arle_gated_delta_scan(const void* q, long long q_stride, const void* k, long long k_stride, const void* v,
                                      long long v_stride, int dtype, const void* gates, long long gates_stride,
                                      const void* a_log, const void* dt_bias, float unit_eps, void* s_state,
-                                     const int* seg_row0, const int* seg_slot, int segments, void* out, int H, int G,
-                                     int D, int Dv, void* stream) {
+                                     const int* seg_row0, const int* seg_slot, int segments, int single_rows, void* out,
+                                     int H, int G, int D, int Dv, void* stream) {
   if (segments == 0) return 0;
   if (D < 1 || D > 256 || H % G) return static_cast<int>(hipErrorInvalidValue);
   dim3 grid(segments, H, (Dv + kGdCols - 1) / kGdCols);
   hipStream_t s = static_cast<hipStream_t>(stream);
 #define ARLE_GD(T, DS)                                                                                               \
-  gated_delta_scan_kernel<T, DS><<<grid, kGdThreads, 0, s>>>(                                                        \
+  if (single_rows) ARLE_GD_L(T, DS, false); else ARLE_GD_L(T, DS, true)
+#define ARLE_GD_L(T, DS, ROWS)                                                                                       \
+  gated_delta_scan_kernel<T, DS, ROWS><<<grid, kGdThreads, 0, s>>>(                                                  \
       static_cast<const T*>(q), q_stride, static_cast<const T*>(k), k_stride, static_cast<const T*>(v), v_stride,    \
       static_cast<const float*>(gates), gates_stride, static_cast<const float*>(a_log),                              \
       static_cast<const float*>(dt_bias), unit_eps, static_cast<float*>(s_state), seg_row0, seg_slot,                \
@@ -178,6 +209,7 @@ extern "C" int arle_gated_delta_scan(const void* q, long long q_stride, const vo
   if (D <= 32) ARLE_GD(T, 2); else if (D <= 64) ARLE_GD(T, 4); else if (D <= 128) ARLE_GD(T, 8); else ARLE_GD(T, 16)
   if (dtype == kF32) { ARLE_GD_T(float); } else { ARLE_GD_T(bf16); }
 #undef ARLE_GD_T
+#undef ARLE_GD_L
 #undef ARLE_GD
   return launch_status();
 }

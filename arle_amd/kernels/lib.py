@@ -88,8 +88,8 @@ SIGNATURES = {
     "arle_pair_norm": ("hyper", [_p, _ll, _i, _ll, _p, _ll, _i, _ll, _i, _p, _p, _f, _f, _p, _i, _i, _i, _p]),
     "arle_rotary_qkv_store": ("rotary_store", [_p, _ll, _p, _ll, _p, _ll, _i, _p, _p, _i, _f, _i, _p, _p, _i, _i, _p, _p,
                                                _p, _i, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
-    "arle_gated_delta_scan": ("gated_delta", [_p, _ll, _p, _ll, _p, _ll, _i, _p, _ll, _p, _p, _f, _p, _p, _p, _i, _p, _i,
-                                              _i, _i, _i, _p]),
+    "arle_gated_delta_scan": ("gated_delta", [_p, _ll, _p, _ll, _p, _ll, _i, _p, _ll, _p, _p, _f, _p, _p, _p, _i, _i, _p,
+                                              _i, _i, _i, _i, _p]),
     "arle_gated_delta_output": ("gated_delta", [_p, _p, _ll, _i, _p, _i, _f, _p, _i, _i, _i, _p]),
     "arle_ceiling_read": ("ceilings", [_p, _ll, _i, _p, _p, _p]),
     "arle_ceiling_mfma": ("ceilings", [_i, _i, _i, _i, _p, _p]),

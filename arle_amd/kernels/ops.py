@@ -2129,7 +2129,8 @@ def gated_delta_scan(q, k, v, gates, a_log, dt_bias, s_state, seg_row0, seg_slot
     out = torch.empty((tokens, H * Dv), dtype=torch.float32, device=q.device)
     lib.call("arle_gated_delta_scan", q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0),
              _code(q), gates.data_ptr(), gates.stride(0), a_log.data_ptr(), dt_bias.data_ptr(), float(unit_eps),
-             s_state.data_ptr(), seg_row0.data_ptr(), seg_slot.data_ptr(), segments, out.data_ptr(), H, G, D, Dv, _stream())
+             s_state.data_ptr(), seg_row0.data_ptr(), seg_slot.data_ptr(), segments, 1 if tokens == segments else 0,
+             out.data_ptr(), H, G, D, Dv, _stream())
     return out
 
 
