@@ -353,8 +353,11 @@ struct CapArgs {
 // HEADS: a work item is one row (a segment of one row) and the q heads of a kv head, and the WAVES waves of the
 // workgroup take its tiles of keys in turn and add their sums through LDS; else an item is sixteen rows of one q head,
 // and the waves of a workgroup are WAVES q heads of one kv head on the same rows, so that they fetch the same tiles.
+// (Portions of heads up to 128 are asked to fit three waves a SIMD: the kernel waits for its loads, and 163 registers
+// hold what 202 held; with larger heads, or four waves, the compiler would spill.)
 template <int KC, int VC, bool HEADS, int WAVES>
-__global__ __launch_bounds__(WAVES * kWave) void attn_softcap_mfma_kernel(const CapArgs a) {
+__global__ __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(!HEADS && KC <= 4 && VC <= 8 ? 3 : 1)))
+void attn_softcap_mfma_kernel(const CapArgs a) {
   extern __shared__ float merge_lds[];   // HEADS: [WAVES][n_vc][64 lanes][4], then m [WAVES][16], l [WAVES][16]; then page ids
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, n = lane % 16, g = lane / 16;
   const int group = a.nq / a.nkv;
@@ -369,8 +372,17 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_softcap_mfma_kernel(const 
     head = kvh * group + min(16 * part + n, group - 1);
     live = 16 * part + n < group;
   } else {
-    // the blockIdx.x-th block of sixteen rows, counted through the segments
-    int left = blockIdx.x, found = -1;
+    // Workgroups go to the chip's eight dies in turn (the launch order is blockIdx.x fastest), and every die has a
+    // level-two cache of its own: with the head groups a multiple of eight, die i takes the head groups i, i + 8, ...
+    // with all their row blocks, so that it keeps the keys and values of its own kv heads and not everybody's.
+    int bx = blockIdx.x, by = blockIdx.y;
+    if (gridDim.y % 8 == 0) {
+      const unsigned linear = blockIdx.y * gridDim.x + blockIdx.x, die = linear % 8, within = linear / 8;
+      by = die + 8 * (within / gridDim.x);
+      bx = within % gridDim.x;
+    }
+    // the bx-th block of sixteen rows, counted through the segments
+    int left = bx, found = -1;
     for (int s = 0; s < a.segments; ++s) {
       const int blocks = (a.seg_row0[s + 1] - a.seg_row0[s] + 15) / 16;
       if (left < blocks) {
@@ -381,7 +393,7 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_softcap_mfma_kernel(const 
     }
     if (found < 0) return;
     seg = found;
-    head = blockIdx.y * WAVES + wave;
+    head = by * WAVES + wave;
     kvh = head / group;
     const int end = a.seg_row0[seg + 1];
     first_row = a.seg_row0[seg] + left * 16;

@@ -181,7 +181,10 @@ ATTENTIONS = [("attention", attn(6, 2, 16, 24, 0.35, 6.0, rot(10000.0, 12)), 4),
               ("sink0", attn(1, 1, 10, 14, 0.6, None, rot(50.0, 6)), 8),
               ("attention_2", attn(6, 3, 16, 8, 0.4, None, rot(3000.0, 16, (4.0, 40, 8.0, 1.0))), 4),
               ("attention_2", attn(4, 2, 64, 64, 0.2, None, rot(250000.0, 64, (2.0, 64, 16.0, 2.0))), 16),
-              ("attention_2", attn(3, 3, 24, 40, 0.3, None, rot(10000.0, 10)), 16)]
+              ("attention_2", attn(3, 3, 24, 40, 0.3, None, rot(10000.0, 10)), 16),
+              # head groups that are a multiple of eight: the matrix-core kernel then deals them to the chip's dies
+              ("sink0", attn(32, 8, 64, 64, 0.2, None, rot(10000.0, 64)), 16),
+              ("attention", attn(16, 16, 32, 32, 0.3, 10.0, rot(100.0, 16)), 16)]
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16])
