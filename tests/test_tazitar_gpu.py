@@ -252,7 +252,7 @@ def delta_part(width, m, dtype, seed, eps=1e-5):
 
 DELTAS = [delta(4, 2, 16, 12), delta(3, 3, 10, 6, conv=2), delta(4, 2, 64, 32, conv=5), delta(5, 1, 40, 10, conv=3),
           delta(2, 1, 24, 20), delta(2, 2, 130, 36, conv=4), delta(1, 1, 8, 70, conv=1),
-          delta(32, 8, 64, 144, conv=2)]      # heads and columns enough for the kernel's form of two columns a wave
+          delta(32, 8, 64, 144, conv=2)]      # many heads over few q/k heads, nine column tiles a head
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16])
