@@ -10,6 +10,9 @@ R: sizes the matrix-core attention takes (keys of 64 and 96, values of 64 and 80
    model inside the loop and run three times, five taps.
 S: two streams, a loop that runs once and one that could be left out (times 1), a loop body of one layer, widths that
    are no multiple of 4, a key size of 40, three taps, no scaling on the interleaved rotation.
+T: sizes of a small real model, on the kernels such a model runs on: heads of 64 and 128 for the matrix cores and the
+   eight-entries-a-lane preparation, sixteen q heads (head groups that are a multiple of eight), a delta rule with key
+   size 128, two streams, the first two layers looped twice, pages of 32.
 """
 from __future__ import annotations
 
@@ -78,9 +81,16 @@ TINY_S = {"architecture": ARCH, "vocab": 150, "width": 54, "norm": {"eps": 1e-5}
                      layer("parallel", {"left": attn(2, 1, 48, 16, scale=0.25, rot=rot(200.0, 48)),
                                         "right": delta(5, 1, 40, 10, conv=3)}, 70)]}
 
+TINY_T = {"architecture": ARCH, "vocab": 500, "width": 256, "norm": {"eps": 1e-6}, "streams": 2,
+          "loop": {"start": 0, "stop": 2, "times": 2},
+          "layers": [layer("parallel", {"left": attn(8, 2, 128, 64, scale=0.09, rot=rot(1000000.0, 64)),
+                                        "right": delta(8, 2, 128, 64, conv=4)}, 384),
+                     layer("attention_2", attn(8, 8, 128, 128, scale=0.09, rot=rot(50000.0, 128, (4.0, 256, 32.0, 1.0))), 384),
+                     layer("attention", attn(16, 4, 64, 64, scale=0.125, softcap=30.0, rot=rot(500000.0, 64)), 384)]}
+
 # name -> (config, page size, weight std, norm std, seed)
 TINY = {"P": (TINY_P, 4, 0.2, 0.2, 5), "Q": (TINY_Q, 8, 0.25, 0.3, 6), "R": (TINY_R, 16, 0.12, 0.2, 7),
-        "S": (TINY_S, 16, 0.2, 0.2, 9)}
+        "S": (TINY_S, 16, 0.2, 0.2, 9), "T": (TINY_T, 32, 0.08, 0.2, 11)}
 
 
 def make_model_dir(tmp_path, name: str) -> str:
