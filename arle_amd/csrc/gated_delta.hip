@@ -77,50 +77,72 @@ __global__ __launch_bounds__(kGdThreads) void gated_delta_scan_kernel(
     const int d = part * DS + i;
     S[i] = (live && d < D) ? s_ptr[static_cast<int64_t>(d) * Dv + col] : 0.f;
   }
+  // A block's rows are fetched from memory into registers while the chain of the block before runs, and go on to LDS
+  // (with their norms and gates) when it has ended.
+  constexpr int kMine = DP / kGdRowThreads;                      // entries of a row's q (and k) a thread prepares
+  constexpr int kValues = kGdRows * kGdCols / kGdThreads;        // entries of the block's v a thread moves
+  const int r = tid / kGdRowThreads, sub = tid % kGdRowThreads;   // a row by kGdRowThreads threads
+  float q_next[kMine], k_next[kMine], v_next[kValues], b_next = 0.f, a_next = 0.f;
+  auto fetch = [&](int base) {
+    const int n = min(kGdRows, rows - base);   // <= 0 behind the last block: nothing is loaded
+    const int64_t t = row0 + base + min(r, max(n, 1) - 1);
+    const T* qr = q + t * q_stride + kvh * D;
+    const T* kr = k + t * k_stride + kvh * D;
+#pragma unroll
+    for (int j = 0; j < kMine; ++j) {
+      const int d = sub + j * kGdRowThreads;
+      const bool there = r < n && d < D;
+      q_next[j] = there ? to_float(qr[d]) : 0.f;
+      k_next[j] = there ? to_float(kr[d]) : 0.f;
+    }
+    if (sub == 0 && r < n) {
+      b_next = gates[t * gates_stride + h];
+      a_next = gates[t * gates_stride + H + h];
+    }
+#pragma unroll
+    for (int j = 0; j < kValues; ++j) {
+      const int e = tid + j * kGdThreads, rr = e / kGdCols, cc = e % kGdCols;
+      const int c_abs = min(static_cast<int>(blockIdx.z) * kGdCols + cc, Dv - 1);
+      v_next[j] = rr < n ? to_float(v[(row0 + base + rr) * v_stride + h * Dv + c_abs]) : 0.f;
+    }
+  };
+  fetch(0);
   for (int base = 0; base < rows; base += kGdRows) {
     const int n = min(kGdRows, rows - base);
     __syncthreads();   // the block before has been read
-    {   // a row by kGdRowThreads threads: its q and k to LDS, their unit norms, k . q, the gates
-      const int r = tid / kGdRowThreads, sub = tid % kGdRowThreads;
-      const int64_t t = row0 + base + min(r, n - 1);
-      if (r < n) {   // (the threads of a row leave or stay together; a decoded row's block is one row)
-        const T* qr = q + t * q_stride + kvh * D;
-        const T* kr = k + t * k_stride + kvh * D;
-        float sq = 0.f, sk = 0.f, kq = 0.f;
-        for (int d = sub; d < DP; d += kGdRowThreads) {
-          const float qv = d < D ? to_float(qr[d]) : 0.f, kv = d < D ? to_float(kr[d]) : 0.f;
-          q_lds[r][d] = qv;
-          k_lds[r][d] = kv;
-          sq = fmaf(qv, qv, sq);
-          sk = fmaf(kv, kv, sk);
-          kq = fmaf(kv, qv, kq);
-        }
+    if (r < n) {   // (the threads of a row leave or stay together; a decoded row's block is one row)
+      float sq = 0.f, sk = 0.f, kq = 0.f;
 #pragma unroll
-        for (int off = kGdRowThreads / 2; off > 0; off >>= 1) {
-          sq += __shfl_xor(sq, off, kWave);
-          sk += __shfl_xor(sk, off, kWave);
-          kq += __shfl_xor(kq, off, kWave);
-        }
-        const float fq = q_scale / sqrtf(sq + unit_eps), fk = 1.0f / sqrtf(sk + unit_eps);
-        for (int d = sub; d < DP; d += kGdRowThreads) {   // the entries this thread has written itself
-          q_lds[r][d] *= fq;
-          k_lds[r][d] *= fk;
-        }
-        if (sub == 0) {
-          const float b = gates[t * gates_stride + h], a = gates[t * gates_stride + H + h];
-          c_lds[r][0] = expf(-rate * softplus(a + bias));
-          c_lds[r][1] = 1.0f / (1.0f + expf(-b));
-          c_lds[r][2] = kq * fq * fk;
-        }
+      for (int j = 0; j < kMine; ++j) {
+        sq = fmaf(q_next[j], q_next[j], sq);
+        sk = fmaf(k_next[j], k_next[j], sk);
+        kq = fmaf(k_next[j], q_next[j], kq);
       }
-      for (int e = tid; e < n * kGdCols; e += kGdThreads) {
-        const int rr = e / kGdCols, cc = e % kGdCols;
-        const int64_t tt = row0 + base + min(rr, n - 1);
-        const int c_abs = min(static_cast<int>(blockIdx.z) * kGdCols + cc, Dv - 1);
-        v_lds[rr][cc] = to_float(v[tt * v_stride + h * Dv + c_abs]);
+#pragma unroll
+      for (int off = kGdRowThreads / 2; off > 0; off >>= 1) {
+        sq += __shfl_xor(sq, off, kWave);
+        sk += __shfl_xor(sk, off, kWave);
+        kq += __shfl_xor(kq, off, kWave);
+      }
+      const float fq = q_scale / sqrtf(sq + unit_eps), fk = 1.0f / sqrtf(sk + unit_eps);
+#pragma unroll
+      for (int j = 0; j < kMine; ++j) {
+        q_lds[r][sub + j * kGdRowThreads] = q_next[j] * fq;
+        k_lds[r][sub + j * kGdRowThreads] = k_next[j] * fk;
+      }
+      if (sub == 0) {
+        c_lds[r][0] = expf(-rate * softplus(a_next + bias));
+        c_lds[r][1] = 1.0f / (1.0f + expf(-b_next));
+        c_lds[r][2] = kq * fq * fk;
       }
     }
+#pragma unroll
+    for (int j = 0; j < kValues; ++j) {
+      const int e = tid + j * kGdThreads;
+      v_lds[e / kGdCols][e % kGdCols] = v_next[j];
+    }
     __syncthreads();
+    fetch(base + kGdRows);
     for (int r = 0; r < n; ++r) {
       const float g = c_lds[r][0], beta = c_lds[r][1], kq = c_lds[r][2];
       float kk[DS], dk = 0.f, dq = 0.f;
