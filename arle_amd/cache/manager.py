@@ -64,6 +64,7 @@ class PagedNeed:
     head_dim: int = 0
     window: int | None = None  # None: every earlier token is kept
     chunk: int | None = None   # queries read only the keys of their own chunk of so many positions; None: no chunks
+    keep_first: int = 0        # with a window: the request's first so many keys stay readable behind it
     tensors: tuple = ()        # of PageTensor; empty: "k" [kv_heads, PAGE, head_dim] and "v" [kv_heads, head_dim, PAGE]
     page_size: int | None = None   # tokens a page of this need holds; None: the manager's own page length
 
@@ -226,7 +227,7 @@ class CacheManager:
                     self._group_needs.append(need)
                     self._group_entries.append([])
                     self.groups.append(PageGroup(num_pages if own == page_size else (num_pages * page_size) // own,
-                                                 own, need.window, need.chunk))
+                                                 own, need.window, need.chunk, need.keep_first))
                 g = self._group_needs.index(need)
                 self._entry_place[entry] = (g, len(self._group_entries[g]))
                 self._group_entries[g].append(entry)

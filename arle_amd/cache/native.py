@@ -17,6 +17,7 @@ _SIGNATURES = {
     "arle_group_create": (_p, [_i, _i, _i]),
     "arle_group_destroy": (None, [_p]),
     "arle_group_set_chunk": (_i, [_p, _i]),
+    "arle_group_set_keep_first": (_i, [_p, _i]),
     "arle_group_num_pages": (_i, [_p]),
     "arle_group_free_count": (_i, [_p]),
     "arle_group_held_count": (_i, [_p]),

@@ -96,9 +96,13 @@ class PageGroup:
     The bookkeeping lives in the native runtime core; request keys (any hashable) are mapped to
     integers here."""
 
-    def __init__(self, num_pages: int, page_size: int, window: int | None = None, chunk: int | None = None):
+    def __init__(self, num_pages: int, page_size: int, window: int | None = None, chunk: int | None = None,
+                 keep_first: int = 0):
         """chunk: queries read only the keys of their own chunk of so many positions (counted from position 0), so the
-        pages in front of the newest chunk go back like those a window has passed."""
+        pages in front of the newest chunk go back like those a window has passed.  keep_first: queries still read the
+        request's first so many keys behind the window, so the pages that hold them never go back."""
+        if keep_first < 0:
+            raise ValueError("keep_first must not be negative")
         if page_size <= 0:
             raise ValueError("page_size must be positive")
         if window is not None and window <= 0:
@@ -114,6 +118,9 @@ class PageGroup:
         self._h = self._lib.arle_group_create(num_pages, page_size, window or 0)
         if chunk is not None:
             self._lib.arle_group_set_chunk(self._h, int(chunk))
+        self.keep_first = int(keep_first)
+        if keep_first:
+            self._lib.arle_group_set_keep_first(self._h, int(keep_first))
         self.pool = PagePool(num_pages, _handle=self._h)
         self._ids: dict = {}     # request key -> native id
         self._next_id = 0

@@ -79,7 +79,7 @@ __global__ __launch_bounds__(kWave) void attn_softcap_simt_kernel(
     const T* __restrict__ v_pages, const int* __restrict__ block_table, int table_stride,
     const int* __restrict__ positions, const int* __restrict__ slot_of_token, int nq, int nkv, int Dk, int Dv,
     int page_size, float scale, float cap, const void* __restrict__ r1, const void* __restrict__ r2, int r_dtype,
-    int window, int chunk, const void* __restrict__ sink, int sink_dtype) {
+    int window, int chunk, const void* __restrict__ sink, int sink_dtype, int keep_first) {
   extern __shared__ float qs[];  // [Dk]
   const int t = blockIdx.x;
   const int h = blockIdx.y;
@@ -96,7 +96,11 @@ __global__ __launch_bounds__(kWave) void attn_softcap_simt_kernel(
   __syncthreads();
 
   int first = window > 0 ? max(0, pos - window + 1) : 0;
-  if (chunk > 0) first = max(first, pos / chunk * chunk);
+  // the first `kept` keys of the request stay visible when the window has passed them (the chunk rule still holds)
+  const int chunk_first = chunk > 0 ? pos / chunk * chunk : 0;
+  first = max(first, chunk_first);
+  const int kept = min(keep_first, first);              // keys [chunk_first, kept) and [first, pos] are seen
+  const bool head_part = kept > chunk_first;
   const int64_t k_page = static_cast<int64_t>(nkv) * page_size * Dk, v_page = static_cast<int64_t>(nkv) * page_size * Dv;
   const int64_t k_head = static_cast<int64_t>(kvh) * page_size * Dk, v_head = static_cast<int64_t>(kvh) * page_size * Dv;
 
@@ -105,9 +109,13 @@ __global__ __launch_bounds__(kWave) void attn_softcap_simt_kernel(
 #pragma unroll
   for (int i = 0; i < kCapMaxD / kWave; ++i) acc[i] = 0.f;
 
-  for (int tile = first / kWave; tile * kWave <= pos; ++tile) {
+  for (int tile = head_part ? chunk_first / kWave : first / kWave; tile * kWave <= pos; ++tile) {
+    if (head_part && tile * kWave >= kept && (tile + 1) * kWave <= first) {   // a tile between the two parts
+      tile = first / kWave - 1;
+      continue;
+    }
     const int c = tile * kWave + lane;
-    const bool valid = c >= first && c <= pos;
+    const bool valid = c <= pos && (c >= first || (head_part && c >= chunk_first && c < kept));
     float s = -INFINITY;
     if (valid) {
       const int page = table[c / page_size];
@@ -125,11 +133,12 @@ __global__ __launch_bounds__(kWave) void attn_softcap_simt_kernel(
 #pragma unroll
     for (int i = 0; i < kCapMaxD / kWave; ++i) acc[i] *= alpha;
 
-    const int j_lo = max(first - tile * kWave, 0);
+    const int j_lo = max((head_part ? chunk_first : first) - tile * kWave, 0);
     const int j_hi = min(pos - tile * kWave, kWave - 1);
     for (int j = j_lo; j <= j_hi; ++j) {
       const float pj = __shfl(p, j, kWave);
       const int cj = tile * kWave + j;
+      if (cj < first && cj >= kept) continue;   // between the parts: a page that may have been given back
       const int page = table[cj / page_size];
       const T* vr = v_pages + page * v_page + v_head + (cj % page_size);  // [d][slot in page]
 #pragma unroll
@@ -169,15 +178,51 @@ __global__ __launch_bounds__(kWideThreads) void wide_norm_store_kernel(
     long long v_stride, const T* __restrict__ v_first, long long vf_stride, const void* __restrict__ q_weight,
     const void* __restrict__ k_weight, int w_dtype, const void* __restrict__ lambda, int lambda_dtype, float eps,
     const int* __restrict__ positions, const int* __restrict__ slot_of_token, const int* __restrict__ block_table,
-    int table_stride, T* __restrict__ k_pages, T* __restrict__ v_pages, int nq, int nkv, int Dk, int Dv, int page_size) {
+    int table_stride, T* __restrict__ k_pages, T* __restrict__ v_pages, int nq, int nkv, int Dk, int Dv, int page_size,
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot, int halves) {
+  extern __shared__ float staged[];   // [max(nq, nkv) * Dk] with a rotation, else nothing
   __shared__ float lds[kWideThreads / kWave];
   const int64_t t = blockIdx.x;
   const int what = blockIdx.y;
   const int pos = positions[t];
+  // With a rotation the normed row waits in LDS, so that an entry's partner is read as it was before anything is
+  // written: entry d < rot of a head turns with entry d ^ 1 (or, with `halves`, d +- rot / 2) by the angle of its pair.
+  const int half = rot / 2;
+  const float* cs = rot ? cos_t + static_cast<int64_t>(pos) * half : nullptr;
+  const float* sn = rot ? sin_t + static_cast<int64_t>(pos) * half : nullptr;
+  auto turned = [&](const float* head, int d) {
+    const int partner = halves ? (d < half ? d + half : d - half) : (d ^ 1);
+    const int pair = halves ? (d < half ? d : d - half) : d / 2;
+    const bool second = halves ? d >= half : (d & 1);
+    const float c = cs[pair], sv = sn[pair];
+    return second ? fmaf(head[d], c, head[partner] * sv) : fmaf(head[d], c, -head[partner] * sv);
+  };
+  auto stage = [&](const T* row, int width, const void* weight) {   // the row, normed where it has a weight, into LDS
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < width; i += kWideThreads) {
+      const float x = to_float(row[i]);
+      staged[i] = x;
+      ss = fmaf(x, x, ss);
+    }
+    const float total = block_sum<kWideThreads / kWave>(ss, lds);   // (its barriers also order the writes above)
+    if (weight) {
+      const float inv = 1.0f / sqrtf(total / static_cast<float>(width) + eps);
+      for (int i = threadIdx.x; i < width; i += kWideThreads) staged[i] = staged[i] * inv * load_as_float(weight, w_dtype, i);
+    }
+    __syncthreads();
+  };
   if (what == 0) {
-    if (!q_weight) return;
+    if (!q_weight && !rot) return;
     const int width = nq * Dk;
     T* row = q + t * q_stride;
+    if (rot) {
+      stage(row, width, q_weight);
+      for (int i = threadIdx.x; i < width; i += kWideThreads) {
+        const int d = i % Dk;
+        row[i] = from_float<T>(d < rot ? turned(staged + (i - d), d) : staged[i]);
+      }
+      return;
+    }
     float ss = 0.f;
     for (int i = threadIdx.x; i < width; i += kWideThreads) {
       const float x = to_float(row[i]);
@@ -193,6 +238,15 @@ __global__ __launch_bounds__(kWideThreads) void wide_norm_store_kernel(
   if (what == 1) {
     const int width = nkv * Dk;
     const T* row = k + t * k_stride;
+    if (rot) {
+      stage(row, width, k_weight);
+      for (int i = threadIdx.x; i < width; i += kWideThreads) {
+        const int g = i / Dk, d = i % Dk;
+        k_pages[((page * nkv + g) * page_size + in_page) * Dk + d] =
+            from_float<T>(d < rot ? turned(staged + (i - d), d) : staged[i]);
+      }
+      return;
+    }
     float inv = 1.0f;
     if (k_weight) {
       float ss = 0.f;
@@ -257,9 +311,10 @@ extern "C" int arle_attn_softcap_simt(const void* q, long long q_stride, void* o
                                       int table_stride, const int* positions, const int* slot_of_token, int tokens,
                                       int nq, int nkv, int Dk, int Dv, int page_size, float scale, float cap,
                                       const void* r1, const void* r2, int r_dtype, int window, int chunk,
-                                      const void* sink, int sink_dtype, void* stream) {
+                                      const void* sink, int sink_dtype, int keep_first, void* stream) {
   if (tokens == 0) return 0;
-  if (Dk > kCapMaxD || Dv > kCapMaxD || nkv < 1 || nq % nkv != 0 || nq > 65535 || window < 0 || chunk < 0)
+  if (Dk > kCapMaxD || Dv > kCapMaxD || nkv < 1 || nq % nkv != 0 || nq > 65535 || window < 0 || chunk < 0 ||
+      keep_first < 0 || (keep_first > 0 && window == 0))
     return static_cast<int>(hipErrorInvalidValue);
   hipStream_t s = static_cast<hipStream_t>(stream);
   dim3 grid(tokens, nq);
@@ -268,41 +323,59 @@ extern "C" int arle_attn_softcap_simt(const void* q, long long q_stride, void* o
     attn_softcap_simt_kernel<float><<<grid, kWave, lds, s>>>(
         static_cast<const float*>(q), q_stride, static_cast<float*>(out), o_stride, static_cast<const float*>(k_pages),
         static_cast<const float*>(v_pages), block_table, table_stride, positions, slot_of_token, nq, nkv, Dk, Dv,
-        page_size, scale, cap, r1, r2, r_dtype, window, chunk, sink, sink_dtype);
+        page_size, scale, cap, r1, r2, r_dtype, window, chunk, sink, sink_dtype, keep_first);
   } else {
     attn_softcap_simt_kernel<bf16><<<grid, kWave, lds, s>>>(
         static_cast<const bf16*>(q), q_stride, static_cast<bf16*>(out), o_stride, static_cast<const bf16*>(k_pages),
         static_cast<const bf16*>(v_pages), block_table, table_stride, positions, slot_of_token, nq, nkv, Dk, Dv,
-        page_size, scale, cap, r1, r2, r_dtype, window, chunk, sink, sink_dtype);
+        page_size, scale, cap, r1, r2, r_dtype, window, chunk, sink, sink_dtype, keep_first);
   }
   return launch_status();
 }
 
 // q [T, nq*Dk] is normed in place over the whole row (q_weight [nq*Dk] or null); k [T, nkv*Dk] is normed likewise
 // (k_weight [nkv*Dk] or null) and goes to the pages; v [T, nkv*Dv], mixed with v_first by *lambda where v_first is
-// given, goes to the pages.
+// given, goes to the pages.  rot > 0: behind the norm the first `rot` entries of every head of q and k turn by the
+// angles of float32 tables cos, sin [positions, rot / 2]; halves != 0 pairs entry i with i + rot / 2, else 2i with 2i + 1.
 extern "C" int arle_wide_norm_store(void* q, long long q_stride, const void* k, long long k_stride, const void* v,
                                     long long v_stride, const void* v_first, long long vf_stride, int dtype,
                                     const void* q_weight, const void* k_weight, int w_dtype, const void* lambda,
                                     int lambda_dtype, float eps, const int* positions, const int* slot_of_token,
                                     const int* block_table, int table_stride, void* k_pages, void* v_pages, int tokens,
-                                    int nq, int nkv, int Dk, int Dv, int page_size, void* stream) {
+                                    int nq, int nkv, int Dk, int Dv, int page_size, const float* cos_t,
+                                    const float* sin_t, int rot, int halves, void* stream) {
   if (tokens == 0) return 0;
-  if (nq < 1 || nkv < 1 || Dk < 1 || Dv < 1 || page_size < 1 || (v_first && !lambda)) return static_cast<int>(hipErrorInvalidValue);
+  if (nq < 1 || nkv < 1 || Dk < 1 || Dv < 1 || page_size < 1 || (v_first && !lambda) || rot < 0 || rot > Dk || rot % 2 ||
+      (rot && (!cos_t || !sin_t)))
+    return static_cast<int>(hipErrorInvalidValue);
   const dim3 grid(tokens, 3);
   hipStream_t s = static_cast<hipStream_t>(stream);
+  const size_t staged_bytes = rot ? static_cast<size_t>(nq > nkv ? nq : nkv) * Dk * sizeof(float) : 0;
+  if (staged_bytes > 64 * 1024) return static_cast<int>(hipErrorInvalidValue);
+  if (staged_bytes > 48 * 1024) {
+    static bool raised = false;
+    if (!raised) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&wide_norm_store_kernel<float>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+      if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(&wide_norm_store_kernel<bf16>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+      if (e != hipSuccess) return static_cast<int>(e);
+      raised = true;
+    }
+  }
   if (dtype == kF32) {
-    wide_norm_store_kernel<float><<<grid, kWideThreads, 0, s>>>(
+    wide_norm_store_kernel<float><<<grid, kWideThreads, staged_bytes, s>>>(
         static_cast<float*>(q), q_stride, static_cast<const float*>(k), k_stride, static_cast<const float*>(v), v_stride,
         static_cast<const float*>(v_first), vf_stride, q_weight, k_weight, w_dtype, lambda, lambda_dtype, eps, positions,
         slot_of_token, block_table, table_stride, static_cast<float*>(k_pages), static_cast<float*>(v_pages), nq, nkv, Dk,
-        Dv, page_size);
+        Dv, page_size, cos_t, sin_t, rot, halves);
   } else {
-    wide_norm_store_kernel<bf16><<<grid, kWideThreads, 0, s>>>(
+    wide_norm_store_kernel<bf16><<<grid, kWideThreads, staged_bytes, s>>>(
         static_cast<bf16*>(q), q_stride, static_cast<const bf16*>(k), k_stride, static_cast<const bf16*>(v), v_stride,
         static_cast<const bf16*>(v_first), vf_stride, q_weight, k_weight, w_dtype, lambda, lambda_dtype, eps, positions,
         slot_of_token, block_table, table_stride, static_cast<bf16*>(k_pages), static_cast<bf16*>(v_pages), nq, nkv, Dk,
-        Dv, page_size);
+        Dv, page_size, cos_t, sin_t, rot, halves);
   }
   return launch_status();
 }
@@ -347,6 +420,7 @@ struct CapArgs {
   int chunk;                          // 0: none; else a row sees only the keys of its own chunk of so many positions
   const void* sink; int sink_dtype;   // [nq] or null: exp(sink_h) joins the softmax's denominator
   int merge_floats;   // floats of dynamic LDS in front of the page ids
+  int keep_first;     // with a window: the request's first so many keys stay visible behind it (0: none)
 };
 
 // KC: chunks of 32 of the key size held (Dk <= 32 KC); VC: chunks of 16 of the value size (Dv <= 16 VC).
@@ -413,6 +487,13 @@ void attn_softcap_mfma_kernel(const CapArgs a) {
   };
   const int key_lo = first_seen(pos_lo);
   const int my_lo = first_seen(pos);
+  // The request's first `keep` keys stay visible to rows whose window has passed them.  Their tiles of 32 keys that
+  // lie wholly in front of the first tile of the windows are `head_tiles` tiles of their own, walked first; the walk
+  // counts tiles through both parts (`walk` 0 .. walk_last), and `tile_of` gives the tile of keys behind a count.
+  const int keep = a.keep_first;
+  const int head_tiles = min((keep + 31) / 32, key_lo / 32);
+  const int main_first = key_lo / 32;
+  auto tile_of = [&](int walk) { return walk < head_tiles ? walk : walk - head_tiles + main_first; };
   const float sink = a.sink ? load_as_float(a.sink, a.sink_dtype, head) : -INFINITY;
   const int* table = a.block_table + static_cast<int64_t>(a.seg_slot[seg]) * a.table_stride;
   const float pen1 = a.r1 ? load_as_float(a.r1, a.r_dtype, head) : 0.f;
@@ -436,24 +517,29 @@ void attn_softcap_mfma_kernel(const CapArgs a) {
   const int64_t k_page = static_cast<int64_t>(a.nkv) * a.page_size * a.Dk, v_page = static_cast<int64_t>(a.nkv) * a.page_size * a.Dv;
   const int64_t k_head = static_cast<int64_t>(kvh) * a.page_size * a.Dk, v_head = static_cast<int64_t>(kvh) * a.page_size * a.Dv;
   const int tile_step = HEADS ? WAVES : 1;
-  const int tile_first = key_lo / 32 + (HEADS ? wave : 0);
-  const int tile_last = pos_hi / 32, last_entry = a.table_stride - 1;
+  const int tile_first = HEADS ? wave : 0;                                   // counts of the walk
+  const int tile_last = head_tiles + pos_hi / 32 - main_first, last_entry = a.table_stride - 1;
 
   // Every load of a tile (K rows, V columns, after the two page ids) is sent a tile ahead, while the tile before it
   // is worked through; a tile past the last is the last one again, fetched and dropped.
   // The ids of the pages that the item sees are put into LDS once: a tile's loads then follow no load of a page id,
   // and the reads of LDS are counted apart from the loads from memory, so they disturb no wait for those.
   const int page_first = (key_lo / 32 * 32) / a.page_size;   // the page of the first tile's first key, which may lie in front of key_lo's
-  int* page_lds = reinterpret_cast<int*>(merge_lds) + a.merge_floats;
-  for (int i = threadIdx.x; i <= (tile_last * 32 + 31) / a.page_size - page_first; i += WAVES * kWave)
+  // (the ids of the head tiles' pages, the request's first ones, lie in front of them)
+  const int head_pages = head_tiles > 0 ? (head_tiles * 32 + a.page_size - 1) / a.page_size : 0;
+  int* head_lds = reinterpret_cast<int*>(merge_lds) + a.merge_floats;
+  int* page_lds = head_lds + head_pages;
+  for (int i = threadIdx.x; i < head_pages; i += WAVES * kWave) head_lds[i] = table[min(i, last_entry)];
+  for (int i = threadIdx.x; i <= (pos_hi / 32 * 32 + 31) / a.page_size - page_first; i += WAVES * kWave)
     page_lds[i] = table[min(page_first + i, last_entry)];
   __syncthreads();
-  auto load_tile = [&](int tile, u32x4_t (&kraw)[2][KC], u32x4_t (&vraw)[VC]) {
-    const int key0 = min(tile, tile_last) * 32;
+  auto load_tile = [&](int walk, u32x4_t (&kraw)[2][KC], u32x4_t (&vraw)[VC]) {
+    const int at = min(walk, tile_last);
+    const int key0 = tile_of(at) * 32;
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       const int kb = key0 + 16 * half;
-      const int64_t page = max(page_lds[max(kb / a.page_size - page_first, 0)], 0);
+      const int64_t page = max(at < head_tiles ? head_lds[kb / a.page_size] : page_lds[max(kb / a.page_size - page_first, 0)], 0);
       const int in_page = kb % a.page_size;
       const bf16* kr = a.k_pages + page * k_page + k_head + static_cast<int64_t>(in_page + n) * a.Dk;
       // no load stands under a condition (one would make every later wait a wait for all loads in flight): a piece
@@ -474,8 +560,8 @@ void attn_softcap_mfma_kernel(const CapArgs a) {
     }
   };
 
-  auto work_tile = [&](int tile, const u32x4_t (&kraw)[2][KC], const u32x4_t (&vraw)[VC]) {
-    const int key0 = tile * 32;
+  auto work_tile = [&](int walk, const u32x4_t (&kraw)[2][KC], const u32x4_t (&vraw)[VC]) {
+    const int key0 = tile_of(walk) * 32;
     float s[8];
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
@@ -490,7 +576,7 @@ void attn_softcap_mfma_kernel(const CapArgs a) {
         float v = z[i] * a.scale;
         if (a.cap > 0.f) v = a.cap * fast_tanh(v * inv_cap);
         if (a.r1) v -= pen1 * __logf(1.0f + pen2 * static_cast<float>(pos - key));
-        s[4 * half + i] = (key >= my_lo && key <= pos) ? v : -INFINITY;
+        s[4 * half + i] = ((key >= my_lo || key < keep) && key <= pos) ? v : -INFINITY;
       }
     }
     float m_new = m_run;
@@ -517,7 +603,8 @@ void attn_softcap_mfma_kernel(const CapArgs a) {
     pb[2] = pack_bf16x2(p[4], p[5]);
     pb[3] = pack_bf16x2(p[6], p[7]);
     const bf16x8_t pop = __builtin_bit_cast(bf16x8_t, pb);
-    // which of this lane's eight key slots hold written keys (those between the item's first and last key)
+    // which of this lane's eight key slots hold written keys (those between the item's first and last key, and the
+    // kept first ones)
     const bool edge = key0 < key_lo || key0 + 31 > pos_hi;
 #pragma unroll
     for (int c = 0; c < VC; ++c) {
@@ -527,7 +614,7 @@ void attn_softcap_mfma_kernel(const CapArgs a) {
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
             const int key = key0 + 16 * (j / 4) + 4 * g + j % 4;
-            if (key < key_lo || key > pos_hi) vr[j / 2] &= (j % 2) ? 0x0000ffffu : 0xffff0000u;
+            if ((key < key_lo && key >= keep) || key > pos_hi) vr[j / 2] &= (j % 2) ? 0x0000ffffu : 0xffff0000u;
           }
         }
         f32x4_t o = acc[c];
@@ -646,22 +733,23 @@ extern "C" int arle_attn_softcap_mfma(const void* q, long long q_stride, void* o
                                       int segments, int row_blocks, int heads_mode, int nq, int nkv, int Dk, int Dv,
                                       int page_size, float scale, float cap, const void* r1, const void* r2,
                                       int r_dtype, int window, int chunk, const void* sink, int sink_dtype,
-                                      void* stream) {
+                                      int keep_first, void* stream) {
   if (segments == 0) return 0;
+  // (kept first keys go with a window alone: under the chunk rule a row's chunk would have to hold them)
   if (Dk % 8 || Dk > 256 || Dv % 16 || Dv > 256 || page_size % 16 || nkv < 1 || nq % nkv || nq > 65535 ||
-      window < 0 || chunk < 0)
+      window < 0 || chunk < 0 || keep_first < 0 || (keep_first > 0 && (window == 0 || chunk > 0)))
     return static_cast<int>(hipErrorInvalidValue);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const CapArgs a{static_cast<const bf16*>(q), q_stride, static_cast<bf16*>(out), o_stride,
                   static_cast<const bf16*>(k_pages), static_cast<const bf16*>(v_pages), block_table, table_stride,
                   seg_row0, seg_slot, seg_start, segments, nq, nkv, Dk, Dv, page_size, scale, cap, r1, r2, r_dtype, window,
-                  chunk, sink, sink_dtype, heads_mode ? kCapSplitWaves * ((Dv / 16) * kWave * 4 + 32) : 0};
+                  chunk, sink, sink_dtype, heads_mode ? kCapSplitWaves * ((Dv / 16) * kWave * 4 + 32) : 0, keep_first};
   // pages an item can see: its rows' windows (or everything the block table maps) and the tiles' rounding to 32 keys;
   // nothing of a step's lengths, so that a captured launch holds for every later step of its shape
   const long long mapped = static_cast<long long>(table_stride) * page_size;
   const int span = window > 0 && chunk > 0 ? (window < chunk ? window : chunk) : (window > 0 ? window : chunk);
   const long long keys_seen = (span > 0 && span + 16 < mapped ? span + 16 : mapped) + 64;
-  const size_t page_bytes = (static_cast<size_t>(keys_seen) / page_size + 2) * sizeof(int);
+  const size_t page_bytes = (static_cast<size_t>(keys_seen) / page_size + 2 + (keep_first + 31) / page_size + 2) * sizeof(int);
   if (page_bytes > 48 * 1024) return static_cast<int>(hipErrorInvalidValue);
   const int size = (Dk + 1) / 2 > Dv ? (Dk + 1) / 2 : Dv;   // Dk counts half: a chunk of keys is 32 wide, of values 16
   const int group = nq / nkv;

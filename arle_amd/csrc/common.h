@@ -133,7 +133,9 @@ __device__ __forceinline__ void st4<bf16>(bf16* p, float4 v) {
 // The activation of a gated feed-forward's gate, by a code shared with the Python side (the same in every lane).
 constexpr int kActSilu = 0;
 constexpr int kActGeluTanh = 1;   // 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))
+constexpr int kActSigmoid = 2;    // 1 / (1 + exp(-z)): a gate that is not multiplied by its own input
 __device__ __forceinline__ float gate_act(float z, int act) {
+  if (act == kActSigmoid) return 1.0f / (1.0f + expf(-z));
   if (act == kActGeluTanh) return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
   return z / (1.0f + expf(-z));
 }

@@ -179,6 +179,97 @@ extern "C" int arle_sum_partials(const float* parts, int n_parts, long long stri
   return launch_status();
 }
 
+namespace arle {
+
+// out[t, j] = act(gate[t, j]) * x[t, j] for two views with row strides of their own; out is contiguous [T, width].
+template <typename T>
+__global__ void gate_mul_kernel(const T* __restrict__ gate, int64_t gate_stride, const T* __restrict__ x,
+                                int64_t x_stride, T* __restrict__ out, int width, int act_code) {
+  const int64_t t = blockIdx.x;
+  const int j = blockIdx.y * blockDim.x + threadIdx.x;
+  if (j >= width) return;
+  out[t * width + j] = from_float<T>(gate_act(to_float(gate[t * gate_stride + j]), act_code) * to_float(x[t * x_stride + j]));
+}
+
+// bfloat16, eight columns a thread; width and both strides multiples of 8, pointers 16-byte aligned.
+__global__ void gate_mul_bf16x8_kernel(const uint16_t* __restrict__ gate, int64_t gate_stride,
+                                       const uint16_t* __restrict__ x, int64_t x_stride, uint16_t* __restrict__ out,
+                                       int width, int64_t chunks, int act_code) {
+  const int64_t c = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (c >= chunks) return;
+  const int per_row = width / 8;
+  const int64_t t = c / per_row;
+  const int j = static_cast<int>(c % per_row) * 8;
+  const uint4 g4 = *reinterpret_cast<const uint4*>(gate + t * gate_stride + j);
+  const uint4 u4 = *reinterpret_cast<const uint4*>(x + t * x_stride + j);
+  const uint32_t gw[4] = {g4.x, g4.y, g4.z, g4.w}, uw[4] = {u4.x, u4.y, u4.z, u4.w};
+  uint32_t ow[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float g0 = __uint_as_float(gw[i] << 16), g1 = __uint_as_float(gw[i] & 0xffff0000u);
+    const float u0 = __uint_as_float(uw[i] << 16), u1 = __uint_as_float(uw[i] & 0xffff0000u);
+    ow[i] = pack_bf16x2(gate_act(g0, act_code) * u0, gate_act(g1, act_code) * u1);
+  }
+  *reinterpret_cast<uint4*>(out + t * width + j) = uint4{ow[0], ow[1], ow[2], ow[3]};
+}
+
+// out[t, j] = act(z[t, j]) * table[ids[t], first + j]: a gate on a slice of a second embedding's row.
+template <typename T, typename TT>
+__global__ void token_gate_kernel(const T* __restrict__ z, int64_t z_stride, const TT* __restrict__ table,
+                                  int64_t table_stride, int first, const int* __restrict__ ids, T* __restrict__ out,
+                                  int width, int act_code) {
+  const int64_t t = blockIdx.x;
+  const TT* row = table + static_cast<int64_t>(ids[t]) * table_stride + first;
+  for (int j = threadIdx.x; j < width; j += blockDim.x)
+    out[t * width + j] = from_float<T>(gate_act(to_float(z[t * z_stride + j]), act_code) * to_float(row[j]));
+}
+
+}  // namespace arle
+
+// gate, x: [T, width] views of `dtype` with row strides in elements; out contiguous [T, width].  act: a kAct code.
+extern "C" int arle_gate_mul(const void* gate, long long gate_stride, const void* x, long long x_stride, void* out,
+                             int dtype, int tokens, int width, int act, void* stream) {
+  if (tokens == 0 || width == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  if (dtype == kBF16 && width % 8 == 0 && gate_stride % 8 == 0 && x_stride % 8 == 0 && aligned(gate) && aligned(x) &&
+      aligned(out)) {
+    const int64_t chunks = static_cast<int64_t>(tokens) * (width / 8);
+    gate_mul_bf16x8_kernel<<<static_cast<unsigned>((chunks + 255) / 256), 256, 0, s>>>(
+        static_cast<const uint16_t*>(gate), gate_stride, static_cast<const uint16_t*>(x), x_stride,
+        static_cast<uint16_t*>(out), width, chunks, act);
+    return launch_status();
+  }
+  dim3 grid(tokens, (width + 255) / 256);
+  if (dtype == kF32)
+    gate_mul_kernel<float><<<grid, 256, 0, s>>>(static_cast<const float*>(gate), gate_stride, static_cast<const float*>(x),
+                                                x_stride, static_cast<float*>(out), width, act);
+  else
+    gate_mul_kernel<bf16><<<grid, 256, 0, s>>>(static_cast<const bf16*>(gate), gate_stride, static_cast<const bf16*>(x),
+                                               x_stride, static_cast<bf16*>(out), width, act);
+  return launch_status();
+}
+
+// z [T, width] of `dtype` (row stride in elements), table [rows, table_stride] of `table_dtype`, ids int32 [T] (checked
+// by the caller to lie in the table); out contiguous [T, width] of `dtype`.
+extern "C" int arle_token_gate(const void* z, long long z_stride, int dtype, const void* table, long long table_stride,
+                               int table_dtype, int first, const int* ids, void* out, int tokens, int width, int act,
+                               void* stream) {
+  if (tokens == 0 || width == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int threads = width <= 64 ? 64 : 256;
+#define ARLE_TG(T, TT)                                                                                             \
+  token_gate_kernel<T, TT><<<tokens, threads, 0, s>>>(static_cast<const T*>(z), z_stride, static_cast<const TT*>(table), \
+                                                      table_stride, first, ids, static_cast<T*>(out), width, act)
+  if (dtype == kF32) {
+    if (table_dtype == kF32) ARLE_TG(float, float); else ARLE_TG(float, bf16);
+  } else {
+    if (table_dtype == kF32) ARLE_TG(bf16, float); else ARLE_TG(bf16, bf16);
+  }
+#undef ARLE_TG
+  return launch_status();
+}
+
 // x float32 [count], in place.
 extern "C" int arle_tanh_cap(float* x, long long count, float cap, void* stream) {
   if (count == 0) return 0;

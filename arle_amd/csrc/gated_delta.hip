@@ -5,6 +5,8 @@
 //   q <- q / sqrt(sum q^2 + 1e-6) * D^(-1/2),   k <- k / sqrt(sum k^2 + 1e-6)
 //   beta = sigmoid(b),   g = exp(-exp(A_log_h) * softplus(a + dt_bias_h))
 //   S <- g S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q
+// CHANNEL: a decay for every head and key entry, g_d = exp(-exp(A_log_h) * softplus(a_hd + dt_bias_hd)), on the rows of
+// S (S <- diag(g) S); the decays' pre-activations are then a [T, H, D], and dt_bias [H, D].
 // A column of S (one entry of v) never meets another, so the columns spread over workgroups: a workgroup a
 // (request, head, 16 columns), four columns a wave, a sixteenth of D a lane.  Rows go through LDS in blocks of
 // 32; the block's unit norms, gates and the dot products k . q are made there, a row by eight threads, always
@@ -17,7 +19,7 @@
 // time is the state's way in and out): the four columns of a wave are four neighbouring lanes, so that a load of the
 // state is sixteen bytes for every four lanes, and the shares exchange through lane reads four, eight, sixteen and
 // 32 lanes away.  `gated_delta_output` divides each head's o by its root mean square, multiplies by the norm's weight and
-// by silu of the gate's projection.
+// by silu (or sigmoid) of the gate's projection.
 #include "common.h"
 
 namespace arle {
@@ -47,18 +49,20 @@ __device__ __forceinline__ float row16_sum(float v) {
   return v;
 }
 
-template <typename T, int DS, bool ROWS>
+template <typename T, int DS, bool ROWS, bool CHANNEL>
 __global__ __launch_bounds__(kGdThreads) void gated_delta_scan_kernel(
     const T* __restrict__ q, long long q_stride, const T* __restrict__ k, long long k_stride, const T* __restrict__ v,
-    long long v_stride, const float* __restrict__ gates /* [T, >= 2H]: b then a */, long long gates_stride,
+    long long v_stride, const float* __restrict__ beta_in /* [T, H] */, long long beta_stride,
+    const float* __restrict__ decay_in /* [T, H], CHANNEL: [T, H * D] */, long long decay_stride,
     const float* __restrict__ a_log, const float* __restrict__ dt_bias, float unit_eps, float* __restrict__ s_state,
     const int* __restrict__ seg_row0, const int* __restrict__ seg_slot, float* __restrict__ out /* [T, H * Dv] */,
     int H, int G, int D, int Dv) {
   constexpr int DP = kGdParts * DS;   // padded D: what lies past D is zero in LDS and in the registers
   __shared__ __attribute__((aligned(16))) float q_lds[kGdRows][DP];
   __shared__ __attribute__((aligned(16))) float k_lds[kGdRows][DP];
+  __shared__ __attribute__((aligned(16))) float g_lds[CHANNEL ? kGdRows : 1][DP];   // CHANNEL: the decays; q_lds then holds g q
   __shared__ float v_lds[kGdRows][kGdCols];
-  __shared__ float c_lds[kGdRows][4];   // decay, beta, k . q
+  __shared__ float c_lds[kGdRows][4];   // decay (of the head), beta, k . q
   const int seg = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int lane = tid % kWave, wave = tid / kWave;
   const int kvh = h / (H / G);
@@ -69,7 +73,7 @@ __global__ __launch_bounds__(kGdThreads) void gated_delta_scan_kernel(
   const bool live = col < Dv;
   const int row0 = seg_row0[seg], rows = seg_row0[seg + 1] - row0;
   float* s_ptr = s_state + (static_cast<int64_t>(seg_slot[seg]) * H + h) * D * Dv;
-  const float rate = expf(a_log[h]), bias = dt_bias[h], q_scale = 1.0f / sqrtf(static_cast<float>(D));
+  const float rate = expf(a_log[h]), bias = CHANNEL ? 0.f : dt_bias[h], q_scale = 1.0f / sqrtf(static_cast<float>(D));
 
   float S[DS];
 #pragma unroll
@@ -83,6 +87,14 @@ __global__ __launch_bounds__(kGdThreads) void gated_delta_scan_kernel(
   constexpr int kValues = kGdRows * kGdCols / kGdThreads;        // entries of the block's v a thread moves
   const int r = tid / kGdRowThreads, sub = tid % kGdRowThreads;   // a row by kGdRowThreads threads
   float q_next[kMine], k_next[kMine], v_next[kValues], b_next = 0.f, a_next = 0.f;
+  float g_next[CHANNEL ? kMine : 1], g_bias[CHANNEL ? kMine : 1];   // CHANNEL: a_hd of the row, and dt_bias_hd
+  if constexpr (CHANNEL) {
+#pragma unroll
+    for (int j = 0; j < kMine; ++j) {
+      const int d = sub + j * kGdRowThreads;
+      g_bias[j] = d < D ? dt_bias[h * D + d] : 0.f;
+    }
+  }
   auto fetch = [&](int base) {
     const int n = min(kGdRows, rows - base);   // <= 0 behind the last block: nothing is loaded
     const int64_t t = row0 + base + min(r, max(n, 1) - 1);
@@ -94,10 +106,11 @@ __global__ __launch_bounds__(kGdThreads) void gated_delta_scan_kernel(
       const bool there = r < n && d < D;
       q_next[j] = there ? to_float(qr[d]) : 0.f;
       k_next[j] = there ? to_float(kr[d]) : 0.f;
+      if constexpr (CHANNEL) g_next[j] = there ? decay_in[t * decay_stride + h * D + d] : 0.f;
     }
     if (sub == 0 && r < n) {
-      b_next = gates[t * gates_stride + h];
-      a_next = gates[t * gates_stride + H + h];
+      b_next = beta_in[t * beta_stride + h];
+      if constexpr (!CHANNEL) a_next = decay_in[t * decay_stride + h];
     }
 #pragma unroll
     for (int j = 0; j < kValues; ++j) {
@@ -127,11 +140,17 @@ __global__ __launch_bounds__(kGdThreads) void gated_delta_scan_kernel(
       const float fq = q_scale / sqrtf(sq + unit_eps), fk = 1.0f / sqrtf(sk + unit_eps);
 #pragma unroll
       for (int j = 0; j < kMine; ++j) {
-        q_lds[r][sub + j * kGdRowThreads] = q_next[j] * fq;
+        if constexpr (CHANNEL) {   // (past D: a decay of 1 on zeros)
+          const float gd = expf(-rate * softplus(g_next[j] + g_bias[j]));
+          g_lds[r][sub + j * kGdRowThreads] = gd;
+          q_lds[r][sub + j * kGdRowThreads] = q_next[j] * fq * gd;
+        } else {
+          q_lds[r][sub + j * kGdRowThreads] = q_next[j] * fq;
+        }
         k_lds[r][sub + j * kGdRowThreads] = k_next[j] * fk;
       }
       if (sub == 0) {
-        c_lds[r][0] = expf(-rate * softplus(a_next + bias));
+        c_lds[r][0] = CHANNEL ? 1.0f : expf(-rate * softplus(a_next + bias));
         c_lds[r][1] = 1.0f / (1.0f + expf(-b_next));
         c_lds[r][2] = kq * fq * fk;
       }
@@ -145,7 +164,7 @@ __global__ __launch_bounds__(kGdThreads) void gated_delta_scan_kernel(
     fetch(base + kGdRows);
     for (int r = 0; r < n; ++r) {
       const float g = c_lds[r][0], beta = c_lds[r][1], kq = c_lds[r][2];
-      float kk[DS], dk = 0.f, dq = 0.f;
+      float kk[DS], gg[CHANNEL ? DS : 1], dk = 0.f, dq = 0.f;
       if constexpr (DS % 4 == 0) {
         const float4* k4 = reinterpret_cast<const float4*>(&k_lds[r][part * DS]);
         const float4* q4 = reinterpret_cast<const float4*>(&q_lds[r][part * DS]);
@@ -153,6 +172,10 @@ __global__ __launch_bounds__(kGdThreads) void gated_delta_scan_kernel(
         for (int i = 0; i < DS / 4; ++i) {
           const float4 kv = k4[i], qv = q4[i];
           kk[4 * i] = kv.x; kk[4 * i + 1] = kv.y; kk[4 * i + 2] = kv.z; kk[4 * i + 3] = kv.w;
+          if constexpr (CHANNEL) {
+            const float4 gv = reinterpret_cast<const float4*>(&g_lds[r][part * DS])[i];
+            gg[4 * i] = gv.x; gg[4 * i + 1] = gv.y; gg[4 * i + 2] = gv.z; gg[4 * i + 3] = gv.w;
+          }
           dq = fmaf(S[4 * i], qv.x, dq); dq = fmaf(S[4 * i + 1], qv.y, dq);
           dq = fmaf(S[4 * i + 2], qv.z, dq); dq = fmaf(S[4 * i + 3], qv.w, dq);
         }
@@ -160,11 +183,14 @@ __global__ __launch_bounds__(kGdThreads) void gated_delta_scan_kernel(
 #pragma unroll
         for (int i = 0; i < DS; ++i) {
           kk[i] = k_lds[r][part * DS + i];
+          if constexpr (CHANNEL) gg[i] = g_lds[r][part * DS + i];
           dq = fmaf(S[i], q_lds[r][part * DS + i], dq);
         }
       }
+      // CHANNEL: the decayed state is diag(g) S: its products with k and q are S^T (g k) and S^T (g q), the latter
+      // through q_lds, which holds g q
 #pragma unroll
-      for (int i = 0; i < DS; ++i) dk = fmaf(S[i], kk[i], dk);
+      for (int i = 0; i < DS; ++i) dk = fmaf(S[i], CHANNEL ? gg[i] * kk[i] : kk[i], dk);
       if constexpr (ROWS) {   // over the shares of D: with share p ^ 1, then p ^ 2, p ^ 4, p ^ 8
         dk = row16_sum(dk);
         dq = row16_sum(dq);
@@ -177,7 +203,7 @@ __global__ __launch_bounds__(kGdThreads) void gated_delta_scan_kernel(
       }
       const float u = beta * (v_lds[r][col_in] - g * dk);
 #pragma unroll
-      for (int i = 0; i < DS; ++i) S[i] = fmaf(kk[i], u, g * S[i]);
+      for (int i = 0; i < DS; ++i) S[i] = fmaf(kk[i], u, (CHANNEL ? gg[i] : g) * S[i]);
       if (part == 0 && live) out[static_cast<int64_t>(row0 + base + r) * (H * Dv) + h * Dv + col] = fmaf(u, kq, g * dq);
     }
   }
@@ -188,12 +214,12 @@ __global__ __launch_bounds__(kGdThreads) void gated_delta_scan_kernel(
   }
 }
 
-// One wave a (row, head): o / rms(o) * w * silu(gate).
+// One wave a (row, head): o / rms(o) * w * act(gate), act silu or sigmoid (a kAct code).
 template <typename T>
 __global__ __launch_bounds__(kWave) void gated_delta_output_kernel(const float* __restrict__ o, const T* __restrict__ gate,
                                                                    long long gate_stride, const void* __restrict__ weight,
                                                                    int w_dtype, float eps, T* __restrict__ out, int H,
-                                                                   int Dv) {
+                                                                   int Dv, int act) {
   const int64_t t = blockIdx.x;
   const int h = blockIdx.y, lane = threadIdx.x;
   const float* row = o + (t * H + h) * Dv;
@@ -202,7 +228,7 @@ __global__ __launch_bounds__(kWave) void gated_delta_output_kernel(const float* 
   const float inv = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(Dv) + eps);
   for (int d = lane; d < Dv; d += kWave) {
     const float z = to_float(gate[t * gate_stride + h * Dv + d]);
-    out[(t * H + h) * Dv + d] = from_float<T>(row[d] * inv * load_as_float(weight, w_dtype, d) * (z / (1.0f + expf(-z))));
+    out[(t * H + h) * Dv + d] = from_float<T>(row[d] * inv * load_as_float(weight, w_dtype, d) * gate_act(z, act));
   }
 }
 
@@ -211,20 +237,27 @@ __global__ __launch_bounds__(kWave) void gated_delta_output_kernel(const float* 
 using namespace arle;
 
 extern "C" int arle_gated_delta_scan(const void* q, long long q_stride, const void* k, long long k_stride, const void* v,
-                                     long long v_stride, int dtype, const void* gates, long long gates_stride,
-                                     const void* a_log, const void* dt_bias, float unit_eps, void* s_state,
+                                     long long v_stride, int dtype, const void* beta_in, long long beta_stride,
+                                     const void* decay_in, long long decay_stride, const void* a_log, const void* dt_bias, float unit_eps, void* s_state,
                                      const int* seg_row0, const int* seg_slot, int segments, int single_rows, void* out,
-                                     int H, int G, int D, int Dv, void* stream) {
+                                     int H, int G, int D, int Dv, int channel, void* stream) {
   if (segments == 0) return 0;
   if (D < 1 || D > 256 || H % G) return static_cast<int>(hipErrorInvalidValue);
   dim3 grid(segments, H, (Dv + kGdCols - 1) / kGdCols);
   hipStream_t s = static_cast<hipStream_t>(stream);
 #define ARLE_GD(T, DS)                                                                                               \
-  if (single_rows) ARLE_GD_L(T, DS, false); else ARLE_GD_L(T, DS, true)
-#define ARLE_GD_L(T, DS, ROWS)                                                                                       \
-  gated_delta_scan_kernel<T, DS, ROWS><<<grid, kGdThreads, 0, s>>>(                                                  \
+  do {                                                                                                               \
+    if (channel) ARLE_GD_R(T, DS, true); else ARLE_GD_R(T, DS, false);                                               \
+  } while (0)
+#define ARLE_GD_R(T, DS, CH)                                                                                         \
+  do {                                                                                                               \
+    if (single_rows) ARLE_GD_L(T, DS, false, CH); else ARLE_GD_L(T, DS, true, CH);                                   \
+  } while (0)
+#define ARLE_GD_L(T, DS, ROWS, CH)                                                                                   \
+  gated_delta_scan_kernel<T, DS, ROWS, CH><<<grid, kGdThreads, 0, s>>>(                                                \
       static_cast<const T*>(q), q_stride, static_cast<const T*>(k), k_stride, static_cast<const T*>(v), v_stride,    \
-      static_cast<const float*>(gates), gates_stride, static_cast<const float*>(a_log),                              \
+      static_cast<const float*>(beta_in), beta_stride, static_cast<const float*>(decay_in), decay_stride,            \
+      static_cast<const float*>(a_log),                                                                              \
       static_cast<const float*>(dt_bias), unit_eps, static_cast<float*>(s_state), seg_row0, seg_slot,                \
       static_cast<float*>(out), H, G, D, Dv)
 #define ARLE_GD_T(T)                                                                                                 \
@@ -232,22 +265,23 @@ extern "C" int arle_gated_delta_scan(const void* q, long long q_stride, const vo
   if (dtype == kF32) { ARLE_GD_T(float); } else { ARLE_GD_T(bf16); }
 #undef ARLE_GD_T
 #undef ARLE_GD_L
+#undef ARLE_GD_R
 #undef ARLE_GD
   return launch_status();
 }
 
 extern "C" int arle_gated_delta_output(const void* o, const void* gate, long long gate_stride, int dtype,
                                        const void* weight, int w_dtype, float eps, void* out, int tokens, int H, int Dv,
-                                       void* stream) {
+                                       int act, void* stream) {
   if (tokens == 0) return 0;
   dim3 grid(tokens, H);
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (dtype == kF32) {
     gated_delta_output_kernel<float><<<grid, kWave, 0, s>>>(static_cast<const float*>(o), static_cast<const float*>(gate),
-                                                            gate_stride, weight, w_dtype, eps, static_cast<float*>(out), H, Dv);
+                                                            gate_stride, weight, w_dtype, eps, static_cast<float*>(out), H, Dv, act);
   } else {
     gated_delta_output_kernel<bf16><<<grid, kWave, 0, s>>>(static_cast<const float*>(o), static_cast<const bf16*>(gate),
-                                                           gate_stride, weight, w_dtype, eps, static_cast<bf16*>(out), H, Dv);
+                                                           gate_stride, weight, w_dtype, eps, static_cast<bf16*>(out), H, Dv, act);
   }
   return launch_status();
 }

@@ -68,6 +68,7 @@ struct Group {
   int page_size;
   int window;  // 0: none
   int chunk = 0;  // 0: none; else queries read only the keys of their own chunk of so many positions
+  int keep_first = 0;  // with a window: the first so many keys of a request stay readable, so their pages are never trimmed
   Pool pool;
   std::unordered_map<long long, Table> tables;
   Group(int num_pages, int page_size_, int window_) : page_size(page_size_), window(window_), pool(num_pages) {}
@@ -95,6 +96,14 @@ void arle_group_destroy(void* h) { delete G(h); }
 int arle_group_set_chunk(void* h, int chunk) {
   if (chunk < 0) return -1;
   G(h)->chunk = chunk;
+  return 0;
+}
+
+// Queries of this group still read the request's first `keep_first` keys when the window has passed them:
+// `arle_group_trim` leaves the pages that hold them.  0: none.
+int arle_group_set_keep_first(void* h, int keep_first) {
+  if (keep_first < 0) return -1;
+  G(h)->keep_first = keep_first;
   return 0;
 }
 
@@ -190,8 +199,10 @@ int arle_group_trim(void* h, long long key, int* logical, int cap) {
   // the next query sits at position `length`, in the chunk that starts at floor(length / chunk) * chunk
   if (g->chunk > 0) dead = std::max(dead, (t.length / g->chunk * g->chunk) / g->page_size);
   dead = std::min(dead, static_cast<int>(t.pages.size()));
+  // the pages of the kept first keys stay; behind them pages go back as the window passes (first_live counts on from there)
+  const int head = (g->keep_first + g->page_size - 1) / g->page_size;
   int n = 0;
-  for (int i = t.first_live; i < dead; ++i) {
+  for (int i = std::max(t.first_live, head); i < dead; ++i) {
     if (n >= cap) return kBufferTooSmall;
     if (!g->pool.give_back(t.pages[i])) return kNotHeld;
     t.pages[i] = kFreed;

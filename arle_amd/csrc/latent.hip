@@ -8,7 +8,8 @@
 // `latent_prep`: RMS norm of the first C entries of the down projection (plain weight, eps inside the root), the
 // rotation of the R entries behind them and of every head's rotated query part, and the write of [c | k_rot] into
 // the key pages and of c (d-major) into the value pages.  The rotation pairs entry 2i with 2i + 1 over the first
-// `rot` entries, by a table of cos and sin per position; entries past `rot` pass unchanged.
+// `rot` entries (or, with `halves`, entry i with i + rot / 2), by a table of cos and sin per position; entries past
+// `rot` pass unchanged.
 // `head_proj`: out[t, h, :] = in[t, h, :] . Wt[h] for a matrix of its own per head, Wt[h] stored [K, N]; the sum over
 // k is one chain of fused multiply-adds in ascending k for every output, whatever else the launch holds.
 // Norm, angles and sums are 32-bit.
@@ -24,13 +25,21 @@ __global__ __launch_bounds__(kLatentThreads) void latent_prep_kernel(
     T* __restrict__ q_full, long long qf_stride, const void* __restrict__ c_weight, int w_dtype, float eps,
     const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot, const int* __restrict__ positions,
     const int* __restrict__ slot_of_token, const int* __restrict__ block_table, int table_stride,
-    T* __restrict__ k_pages, T* __restrict__ v_pages, int heads, int D, int R, int C, int page_size) {
+    T* __restrict__ k_pages, T* __restrict__ v_pages, int heads, int D, int R, int C, int page_size, int halves) {
   __shared__ float lds[kLatentThreads / kWave];
   const int64_t t = blockIdx.x;
   const int pos = positions[t];
   const int half = rot / 2;
   const float* cs = cos_t + static_cast<int64_t>(pos) * half;
   const float* sn = sin_t + static_cast<int64_t>(pos) * half;
+  // entry i (< rot) of a rotated vector x: x_i cos a -+ x_partner sin a, minus for the first of a pair
+  auto turned = [&](const T* x, int i) {
+    const int partner = halves ? (i < half ? i + half : i - half) : (i ^ 1);
+    const int pair = halves ? (i < half ? i : i - half) : i / 2;
+    const bool second = halves ? i >= half : (i & 1);
+    const float v = to_float(x[i]), other = to_float(x[partner]), c = cs[pair], sv = sn[pair];
+    return second ? fmaf(v, c, other * sv) : fmaf(v, c, -other * sv);
+  };
   if (blockIdx.y == 0) {
     const T* row = dkv + t * dkv_stride;
     float ss = 0.f;
@@ -49,13 +58,7 @@ __global__ __launch_bounds__(kLatentThreads) void latent_prep_kernel(
       vcol[static_cast<int64_t>(i) * page_size] = c;
     }
     for (int i = threadIdx.x; i < R; i += kLatentThreads) {
-      float x = to_float(row[C + i]);
-      if (i < rot) {
-        const float other = to_float(row[C + (i ^ 1)]);
-        const float c = cs[i / 2], s = sn[i / 2];
-        x = (i & 1) ? fmaf(x, c, other * s) : fmaf(x, c, -other * s);
-      }
-      krow[C + i] = from_float<T>(x);
+      krow[C + i] = from_float<T>(i < rot ? turned(row + C, i) : to_float(row[C + i]));
     }
     return;
   }
@@ -63,13 +66,7 @@ __global__ __launch_bounds__(kLatentThreads) void latent_prep_kernel(
   const T* src = q + t * q_stride + static_cast<int64_t>(h) * (D + R) + D;
   T* dst = q_full + t * qf_stride + static_cast<int64_t>(h) * (C + R) + C;
   for (int i = threadIdx.x; i < R; i += kLatentThreads) {
-    float x = to_float(src[i]);
-    if (i < rot) {
-      const float other = to_float(src[i ^ 1]);
-      const float c = cs[i / 2], s = sn[i / 2];
-      x = (i & 1) ? fmaf(x, c, other * s) : fmaf(x, c, -other * s);
-    }
-    dst[i] = from_float<T>(x);
+    dst[i] = from_float<T>(i < rot ? turned(src, i) : to_float(src[i]));
   }
 }
 
@@ -182,7 +179,8 @@ extern "C" int arle_latent_prep(const void* q, long long q_stride, const void* d
                                 long long qf_stride, int dtype, const void* c_weight, int w_dtype, float eps,
                                 const float* cos_t, const float* sin_t, int rot, const int* positions,
                                 const int* slot_of_token, const int* block_table, int table_stride, void* k_pages,
-                                void* v_pages, int tokens, int heads, int D, int R, int C, int page_size, void* stream) {
+                                void* v_pages, int tokens, int heads, int D, int R, int C, int page_size, int halves,
+                                void* stream) {
   if (tokens == 0) return 0;
   if (heads < 1 || heads > 65534 || D < 1 || R < 0 || C < 1 || rot < 0 || rot > R || rot % 2 || page_size < 1 ||
       (rot > 0 && (!cos_t || !sin_t)))
@@ -193,12 +191,12 @@ extern "C" int arle_latent_prep(const void* q, long long q_stride, const void* d
     latent_prep_kernel<float><<<grid, kLatentThreads, 0, s>>>(
         static_cast<const float*>(q), q_stride, static_cast<const float*>(dkv), dkv_stride, static_cast<float*>(q_full),
         qf_stride, c_weight, w_dtype, eps, cos_t, sin_t, rot, positions, slot_of_token, block_table, table_stride,
-        static_cast<float*>(k_pages), static_cast<float*>(v_pages), heads, D, R, C, page_size);
+        static_cast<float*>(k_pages), static_cast<float*>(v_pages), heads, D, R, C, page_size, halves);
   } else {
     latent_prep_kernel<bf16><<<grid, kLatentThreads, 0, s>>>(
         static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(dkv), dkv_stride, static_cast<bf16*>(q_full),
         qf_stride, c_weight, w_dtype, eps, cos_t, sin_t, rot, positions, slot_of_token, block_table, table_stride,
-        static_cast<bf16*>(k_pages), static_cast<bf16*>(v_pages), heads, D, R, C, page_size);
+        static_cast<bf16*>(k_pages), static_cast<bf16*>(v_pages), heads, D, R, C, page_size, halves);
   }
   return launch_status();
 }

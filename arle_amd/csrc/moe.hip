@@ -1,8 +1,11 @@
 // A mixture of experts: the router, and the experts' products over the tokens that chose them.
 //
-//   z = W_r h (32-bit sums),  s = sigmoid(z);  the `top` experts with the largest s + correction are chosen (ties: the
-//   lower index);  weight of a chosen expert = s / (sum of the chosen s + 1e-20) * scale.
-//   expert e: down_e (silu(gate_e h) * (up_e h)).
+//   z = W_r h (32-bit sums),  s = sigmoid(z) or softmax(z) over all router outputs;  the `top` experts with the largest
+//   s + correction are chosen (ties: the lower index), where the experts form `groups` equal groups of neighbours among
+//   the `keep` groups with the largest such number in them only (the others count as minus infinity);  weight of a
+//   chosen expert = s / (sum of the chosen s + 1e-20) * scale, or without the division s * scale.
+//   expert e: down_e (silu(gate_e h) * (up_e h)).  Router outputs past the experts that have tensors stand for experts
+//   that hand back their input (`moe_identity` writes their rows).
 //
 // `moe_route`: one workgroup a token.  `moe_expert`: a workgroup takes one expert, 64 consecutive rows of the step and 64
 // output columns; it lists the rows of its 64 that chose the expert (in row order) and multiplies only those, so no
@@ -39,14 +42,24 @@ constexpr int kRouteThreads = 256;
 // One workgroup a token: the row goes to LDS as floats once; wave w computes the logits of experts w, w + 4, ...
 // (eight consecutive entries a lane and step where the width allows, one otherwise: an order that depends on the
 // width alone); then the first wave picks the `top` experts one after the other.
+struct RouteRule {
+  int softmax;     // 0: s = sigmoid(z); 1: s = softmax(z)
+  int groups;      // equal groups of neighbouring experts (1: no groups)
+  int keep;        // groups among which the choice is made
+  int normalize;   // 1: the chosen scores are divided by their sum
+  float scale;
+};
+
 template <typename T, typename TW, bool VEC>
 __global__ __launch_bounds__(kRouteThreads) void moe_route_kernel(const T* __restrict__ x, long long x_stride,
                                                                   const TW* __restrict__ w, const void* __restrict__ correction,
                                                                   int c_dtype, int* __restrict__ ids, float* __restrict__ weights,
-                                                                  int width, int experts, int top, float scale) {
-  extern __shared__ float route_lds[];   // [width] the row, then [experts] the scores
+                                                                  int width, int experts, int top, const RouteRule rule) {
+  extern __shared__ float route_lds[];   // [width] the row, then [experts] the scores, [experts] the choice numbers, [groups]
   float* xs = route_lds;
   float* score = route_lds + width;
+  float* pick = score + experts;
+  float* group_best = pick + experts;
   const int64_t t = blockIdx.x;
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const T* row = x + t * x_stride;
@@ -65,17 +78,84 @@ __global__ __launch_bounds__(kRouteThreads) void moe_route_kernel(const T* __res
       for (int i = lane; i < width; i += kWave) dot = fmaf(xs[i], to_float(we[i]), dot);
     }
     dot = wave_sum(dot);
-    if (lane == 0) score[e] = 1.0f / (1.0f + expf(-dot));
+    if (lane == 0) score[e] = rule.softmax ? dot : 1.0f / (1.0f + expf(-dot));
   }
   __syncthreads();
-  if (wave != 0) return;
+  // From here on the first wave works alone; the others only keep the barriers' count.
   float s[kMaxExpertsPerLane], choice[kMaxExpertsPerLane];
+  if (wave == 0) {
 #pragma unroll
-  for (int j = 0; j < kMaxExpertsPerLane; ++j) {
-    const int e = lane + j * kWave;
-    s[j] = e < experts ? score[e] : 0.f;
-    choice[j] = e < experts ? s[j] + (correction ? load_as_float(correction, c_dtype, e) : 0.f) : -INFINITY;
+    for (int j = 0; j < kMaxExpertsPerLane; ++j) {
+      const int e = lane + j * kWave;
+      s[j] = e < experts ? score[e] : (rule.softmax ? -INFINITY : 0.f);
+    }
+    if (rule.softmax) {   // over all router outputs, in 32 bits: the largest logit taken off, one sum in a fixed order
+      float top_z = -INFINITY;
+#pragma unroll
+      for (int j = 0; j < kMaxExpertsPerLane; ++j) top_z = fmaxf(top_z, s[j]);
+      top_z = wave_max(top_z);
+      float sum = 0.f;
+#pragma unroll
+      for (int j = 0; j < kMaxExpertsPerLane; ++j) {
+        s[j] = lane + j * kWave < experts ? expf(s[j] - top_z) : 0.f;
+        sum += s[j];
+      }
+      const float inv = 1.0f / wave_sum(sum);
+#pragma unroll
+      for (int j = 0; j < kMaxExpertsPerLane; ++j) s[j] *= inv;
+    }
+#pragma unroll
+    for (int j = 0; j < kMaxExpertsPerLane; ++j) {
+      const int e = lane + j * kWave;
+      choice[j] = e < experts ? s[j] + (correction ? load_as_float(correction, c_dtype, e) : 0.f) : -INFINITY;
+      if (e < experts) pick[e] = choice[j];
+    }
   }
+  if (rule.groups > 1) {   // (the same for every thread of the launch)
+    __syncthreads();
+    const int per = experts / rule.groups;
+    if (wave == 0) {
+      // a group's number is the largest choice number in it; lane l looks after the groups l, l + 64, ...
+      float best[kMaxExpertsPerLane];
+#pragma unroll
+      for (int j = 0; j < kMaxExpertsPerLane; ++j) {
+        const int g = lane + j * kWave;
+        float b = -INFINITY;
+        if (g < rule.groups)
+          for (int i = 0; i < per; ++i) b = fmaxf(b, pick[g * per + i]);
+        best[j] = b;
+        if (g < rule.groups) group_best[g] = 0.f;   // 1 once the group is kept
+      }
+      for (int k = 0; k < rule.keep; ++k) {
+        Best b{-INFINITY, 0x7fffffff};
+#pragma unroll
+        for (int j = 0; j < kMaxExpertsPerLane; ++j) {
+          const int g = lane + j * kWave;
+          if (g < rule.groups && best[j] != INFINITY && (best[j] > b.v || (best[j] == b.v && g < b.i))) {
+            b.v = best[j];
+            b.i = g;
+          }
+        }
+        b = wave_best(b);
+#pragma unroll
+        for (int j = 0; j < kMaxExpertsPerLane; ++j) {
+          if (b.i == lane + j * kWave) {
+            best[j] = INFINITY;   // taken
+            group_best[b.i] = 1.f;
+          }
+        }
+      }
+    }
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+      for (int j = 0; j < kMaxExpertsPerLane; ++j) {
+        const int e = lane + j * kWave;
+        if (e < experts && group_best[e / per] == 0.f) choice[j] = -INFINITY;
+      }
+    }
+  }
+  if (wave != 0) return;
   float sum = 0.f, mine = 0.f;   // lane k keeps the k-th chosen score (top <= 64)
   int mine_id = 0;
   for (int k = 0; k < top; ++k) {
@@ -83,7 +163,7 @@ __global__ __launch_bounds__(kRouteThreads) void moe_route_kernel(const T* __res
 #pragma unroll
     for (int j = 0; j < kMaxExpertsPerLane; ++j) {
       const int e = lane + j * kWave;
-      if (e < experts && (choice[j] > b.v || (choice[j] == b.v && e < b.i))) {
+      if (e < experts && s[j] >= 0.f && (choice[j] > b.v || (choice[j] == b.v && e < b.i))) {
         b.v = choice[j];
         b.i = e;
       }
@@ -95,6 +175,7 @@ __global__ __launch_bounds__(kRouteThreads) void moe_route_kernel(const T* __res
       if (b.i == lane + j * kWave) {
         sv = s[j];
         choice[j] = -INFINITY;
+        s[j] = -1.0f;   // taken: a score is never negative, so this marks it whatever its choice number was
       }
     }
     sv = __shfl(sv, b.i % kWave, kWave);
@@ -106,8 +187,21 @@ __global__ __launch_bounds__(kRouteThreads) void moe_route_kernel(const T* __res
   }
   if (lane < top) {
     ids[t * top + lane] = mine_id;
-    weights[t * top + lane] = mine / (sum + 1e-20f) * scale;
+    weights[t * top + lane] = (rule.normalize ? mine / (sum + 1e-20f) : mine) * rule.scale;
   }
+}
+
+// The rows of experts without tensors: where token t's k-th choice is a router output from `first` on, row t * top + k
+// of out (float32 [T * top, width]) is the token's input itself.  One workgroup a (token, choice).
+template <typename T>
+__global__ __launch_bounds__(256) void moe_identity_kernel(const T* __restrict__ x, long long x_stride,
+                                                           const int* __restrict__ ids, float* __restrict__ out, int top,
+                                                           int width, int first) {
+  const int64_t item = blockIdx.x;
+  if (ids[item] < first) return;
+  const T* row = x + (item / top) * x_stride;
+  float* dst = out + item * width;
+  for (int i = threadIdx.x; i < width; i += 256) dst[i] = to_float(row[i]);
 }
 
 constexpr int kEM = 64, kEN = 64, kEK = 16;
@@ -486,12 +580,15 @@ using namespace arle;
 // float32 [T, top].
 extern "C" int arle_moe_route(const void* x, long long x_stride, int x_dtype, const void* w, int w_dtype,
                               const void* correction, int c_dtype, int* ids, float* weights, int tokens, int width,
-                              int experts, int top, float scale, void* stream) {
+                              int experts, int top, float scale, int softmax, int groups, int keep, int normalize,
+                              void* stream) {
   if (tokens == 0) return 0;
-  if (experts < 1 || experts > kWave * kMaxExpertsPerLane || top < 1 || top > experts || top > kWave)
+  if (experts < 1 || experts > kWave * kMaxExpertsPerLane || top < 1 || top > experts || top > kWave || groups < 1 ||
+      experts % groups || keep < 1 || keep > groups || top > keep * (experts / groups))
     return static_cast<int>(hipErrorInvalidValue);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const size_t lds = static_cast<size_t>(width + experts) * sizeof(float);
+  const RouteRule rule{softmax, groups, keep, normalize, scale};
+  const size_t lds = static_cast<size_t>(width + 2 * experts + groups) * sizeof(float);
   if (lds > 60 * 1024) return static_cast<int>(hipErrorInvalidValue);
   const bool vec = width % 8 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0;
 #define ARLE_ROUTE_V(TX, TWT, V)                                                                                   \
@@ -505,7 +602,7 @@ extern "C" int arle_moe_route(const void* x, long long x_stride, int x_dtype, co
     }                                                                                                              \
     moe_route_kernel<TX, TWT, V><<<tokens, kRouteThreads, lds, s>>>(static_cast<const TX*>(x), x_stride,           \
                                                                     static_cast<const TWT*>(w), correction, c_dtype, \
-                                                                    ids, weights, width, experts, top, scale);      \
+                                                                    ids, weights, width, experts, top, rule);       \
   } while (0)
 #define ARLE_ROUTE(TX, TWT)                          \
   do {                                               \
@@ -519,6 +616,20 @@ extern "C" int arle_moe_route(const void* x, long long x_stride, int x_dtype, co
   }
 #undef ARLE_ROUTE
 #undef ARLE_ROUTE_V
+  return launch_status();
+}
+
+// x [T, width] of `dtype`, ids int32 [T * top], out float32 [T * top, width]: see moe_identity_kernel.
+extern "C" int arle_moe_identity(const void* x, long long x_stride, int dtype, const int* ids, void* out, int tokens,
+                                 int top, int width, int first, void* stream) {
+  if (tokens == 0) return 0;
+  if (top < 1 || width < 1 || first < 0) return static_cast<int>(hipErrorInvalidValue);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const unsigned items = static_cast<unsigned>(tokens) * top;
+  if (dtype == kF32)
+    moe_identity_kernel<float><<<items, 256, 0, s>>>(static_cast<const float*>(x), x_stride, ids, static_cast<float*>(out), top, width, first);
+  else
+    moe_identity_kernel<bf16><<<items, 256, 0, s>>>(static_cast<const bf16*>(x), x_stride, ids, static_cast<float*>(out), top, width, first);
   return launch_status();
 }
 

@@ -1,8 +1,11 @@
 // A norm on a sublayer's output, added into the residual stream:
 //
 //   y_j   = A_j + B_j                           (up to two addends, each a sum of parts, see below)
-//   res_j += y_j / sqrt(mean_j(y_j^2) + eps) * (w_j  or  1 + w_j)
+//   res_j += m * y_j / sqrt(mean_j(y_j^2) + eps) * (w_j  or  1 + w_j)                       (RMS norm), or
+//   res_j += m * ((y_j - mean(y)) / sqrt(mean_j((y_j - mean(y))^2) + eps) * w_j + b_j)        (`center`: layer norm; b optional)
 //   act_j = res_j rounded to the activation type  (what the next sublayer reads; optional)
+//
+// m is one number of the model (1 where it has none).
 //
 // An addend is a float32 tensor [T, W], or parts that are added in ascending order: the float32 partial products of
 // a matrix product whose K was split (part p of row t at p * part_stride + t * row_stride), or the outputs of the
@@ -53,13 +56,14 @@ __device__ __forceinline__ float4 addend_at(const Addend& a, int64_t row, int i)
 template <typename TAct, typename TW, bool VEC>
 __global__ __launch_bounds__(kPostThreads) void norm_add_kernel(float* __restrict__ residual, const Addend a,
                                                                 const Addend b, const TW* __restrict__ w,
-                                                                int one_plus, TAct* __restrict__ act, int width,
+                                                                int one_plus, int center, const TW* __restrict__ bias,
+                                                                float mult, TAct* __restrict__ act, int width,
                                                                 float eps) {
   extern __shared__ float ys[];  // [width]
   __shared__ float lds[kPostWaves];
   const int64_t r = blockIdx.x;
   constexpr int kStep = VEC ? 4 : 1;
-  float ss = 0.f;
+  float ss = 0.f, sum = 0.f;
   for (int i = kStep * threadIdx.x; i < width; i += kStep * kPostThreads) {
     float4 y = addend_at<VEC>(a, r, i);
     if (b.p) {
@@ -69,9 +73,28 @@ __global__ __launch_bounds__(kPostThreads) void norm_add_kernel(float* __restric
     if (VEC) {
       *reinterpret_cast<float4*>(ys + i) = y;
       ss = fmaf(y.x, y.x, ss); ss = fmaf(y.y, y.y, ss); ss = fmaf(y.z, y.z, ss); ss = fmaf(y.w, y.w, ss);
+      sum += (y.x + y.y) + (y.z + y.w);
     } else {
       ys[i] = y.x;
       ss = fmaf(y.x, y.x, ss);
+      sum += y.x;
+    }
+  }
+  float mean = 0.f;
+  if (center) {   // the squares of the deviations from the mean, each thread over the entries it wrote itself
+    mean = block_sum<kPostWaves>(sum, lds) / static_cast<float>(width);
+    ss = 0.f;
+    for (int i = kStep * threadIdx.x; i < width; i += kStep * kPostThreads) {
+      if (VEC) {
+        float4 y = *reinterpret_cast<const float4*>(ys + i);
+        y.x -= mean; y.y -= mean; y.z -= mean; y.w -= mean;
+        *reinterpret_cast<float4*>(ys + i) = y;
+        ss = fmaf(y.x, y.x, ss); ss = fmaf(y.y, y.y, ss); ss = fmaf(y.z, y.z, ss); ss = fmaf(y.w, y.w, ss);
+      } else {
+        const float y = ys[i] - mean;
+        ys[i] = y;
+        ss = fmaf(y, y, ss);
+      }
     }
   }
   const float total = block_sum<kPostWaves>(ss, lds);
@@ -81,13 +104,14 @@ __global__ __launch_bounds__(kPostThreads) void norm_add_kernel(float* __restric
   for (int i = kStep * threadIdx.x; i < width; i += kStep * kPostThreads) {
     if (VEC) {
       const float4 g = ld4<TW>(w + i), y = *reinterpret_cast<const float4*>(ys + i);
+      const float4 c = bias ? ld4<TW>(bias + i) : float4{0.f, 0.f, 0.f, 0.f};
       float4 v = *reinterpret_cast<const float4*>(res + i);
-      v.x = fmaf(y.x * inv, one + g.x, v.x); v.y = fmaf(y.y * inv, one + g.y, v.y);
-      v.z = fmaf(y.z * inv, one + g.z, v.z); v.w = fmaf(y.w * inv, one + g.w, v.w);
+      v.x = fmaf(mult, fmaf(y.x * inv, one + g.x, c.x), v.x); v.y = fmaf(mult, fmaf(y.y * inv, one + g.y, c.y), v.y);
+      v.z = fmaf(mult, fmaf(y.z * inv, one + g.z, c.z), v.z); v.w = fmaf(mult, fmaf(y.w * inv, one + g.w, c.w), v.w);
       *reinterpret_cast<float4*>(res + i) = v;
       if (act) st4<TAct>(act + r * width + i, v);
     } else {
-      const float v = fmaf(ys[i] * inv, one + to_float(w[i]), res[i]);
+      const float v = fmaf(mult, fmaf(ys[i] * inv, one + to_float(w[i]), bias ? to_float(bias[i]) : 0.f), res[i]);
       res[i] = v;
       if (act) act[r * width + i] = from_float<TAct>(v);
     }
@@ -99,11 +123,12 @@ __global__ __launch_bounds__(kPostThreads) void norm_add_kernel(float* __restric
 using namespace arle;
 
 // residual float32 [rows, width], updated in place.  Addends are float32.  act: [rows, width] of act_dtype, or null.
+// center != 0: the layer norm; bias: [width] of the weight's type, or null; mult: the factor on what is added.
 extern "C" int arle_norm_add(float* residual, const float* a, int a_parts, long long a_part_stride,
                              long long a_row_stride, const float* a_weights, const float* b, int b_parts,
                              long long b_part_stride, long long b_row_stride, const float* b_weights,
-                             const void* w, int w_dtype, int one_plus, void* act, int act_dtype, int rows, int width,
-                             float eps, void* stream) {
+                             const void* w, int w_dtype, int one_plus, int center, const void* bias, float mult,
+                             void* act, int act_dtype, int rows, int width, float eps, void* stream) {
   if (rows == 0) return 0;
   if (!a || a_parts < 1 || (b && b_parts < 1) || width < 1 || width > 16384) return static_cast<int>(hipErrorInvalidValue);
   const Addend A{a, a_parts, a_part_stride, a_row_stride, a_weights};
@@ -112,7 +137,7 @@ extern "C" int arle_norm_add(float* residual, const float* a, int a_parts, long 
   const size_t lds = static_cast<size_t>(width) * sizeof(float);
   auto al = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
   const bool vec = width % 4 == 0 && al(residual) && al(a) && a_part_stride % 4 == 0 && a_row_stride % 4 == 0 &&
-                   (!b || (al(b) && b_part_stride % 4 == 0 && b_row_stride % 4 == 0)) && al(w) && al(act);
+                   (!b || (al(b) && b_part_stride % 4 == 0 && b_row_stride % 4 == 0)) && al(w) && al(act) && al(bias);
 #define ARLE_POST_V(TA, TWT, V)                                                                                \
   do {                                                                                                         \
     static bool raised = false;                                                                                \
@@ -123,7 +148,8 @@ extern "C" int arle_norm_add(float* residual, const float* a, int a_parts, long 
       raised = true;                                                                                           \
     }                                                                                                          \
     norm_add_kernel<TA, TWT, V><<<rows, kPostThreads, lds, s>>>(residual, A, B, static_cast<const TWT*>(w),    \
-                                                                one_plus, static_cast<TA*>(act), width, eps);  \
+                                                                one_plus, center, static_cast<const TWT*>(bias), \
+                                                                mult, static_cast<TA*>(act), width, eps);      \
   } while (0)
 #define ARLE_POST(TA, TWT)                     \
   do {                                         \

@@ -58,7 +58,7 @@ SIGNATURES = {
     "arle_attn_decode_static": ("attention_mfma", [_p, _ll, _p, _ll, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i,
                                                    _i, _f, _i, _i, _p]),
     "arle_add_layernorm": ("layernorm", [_p, _p, _i, _ll, _i, _p, _i, _p, _i, _ll, _i, _p, _i, _p, _p, _i, _p, _p, _i, _p, _i,
-                                         _i, _f, _p]),
+                                         _i, _f, _p, _p, _p]),
     "arle_causal_conv": ("short_conv", [_p, _ll, _i, _p, _i, _p, _i, _p, _i, _p, _p, _ll, _i, _i, _i, _i, _i, _p]),
     "arle_conv_state_update": ("short_conv", [_p, _ll, _i, _p, _i, _p, _i, _p, _p, _i, _i, _i, _p]),
     "arle_polynorm": ("polynorm", [_p, _ll, _i, _p, _i, _p, _i, _p, _i, _i, _i, _f, _p]),
@@ -68,29 +68,33 @@ SIGNATURES = {
     "arle_qkv_norm_store": ("attention_softcap", [_p, _ll, _p, _ll, _p, _ll, _i, _p, _p, _i, _f, _f, _i, _p, _p, _p, _i,
                                                   _p, _p, _i, _i, _i, _i, _i, _i, _p]),
     "arle_attn_softcap_simt": ("attention_softcap", [_p, _ll, _p, _ll, _p, _p, _i, _p, _i, _p, _p, _i, _i, _i, _i, _i, _i,
-                                                     _f, _f, _p, _p, _i, _i, _i, _p, _i, _p]),
+                                                     _f, _f, _p, _p, _i, _i, _i, _p, _i, _i, _p]),
     "arle_attn_softcap_mfma": ("attention_softcap", [_p, _ll, _p, _ll, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i,
-                                                     _i, _f, _f, _p, _p, _i, _i, _i, _p, _i, _p]),
+                                                     _i, _f, _f, _p, _p, _i, _i, _i, _p, _i, _i, _p]),
     "arle_attn_softcap_lds_limit": ("attention_softcap", []),
     "arle_wide_norm_store": ("attention_softcap", [_p, _ll, _p, _ll, _p, _ll, _p, _ll, _i, _p, _p, _i, _p, _i, _f, _p, _p,
-                                                   _p, _i, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
+                                                   _p, _i, _p, _p, _i, _i, _i, _i, _i, _i, _p, _p, _i, _i, _p]),
     "arle_tanh_cap": ("elementwise", [_p, _ll, _f, _p]),
-    "arle_norm_add": ("post_norm", [_p, _p, _i, _ll, _ll, _p, _p, _i, _ll, _ll, _p, _p, _i, _i, _p, _i, _i, _i, _f, _p]),
+    "arle_norm_add": ("post_norm", [_p, _p, _i, _ll, _ll, _p, _p, _i, _ll, _ll, _p, _p, _i, _i, _i, _p, _f, _p, _i, _i, _i, _f,
+                                    _p]),
     "arle_latent_prep": ("latent", [_p, _ll, _p, _ll, _p, _ll, _i, _p, _i, _f, _p, _p, _i, _p, _p, _p, _i, _p, _p, _i, _i,
-                                    _i, _i, _i, _i, _p]),
+                                    _i, _i, _i, _i, _i, _p]),
     "arle_head_proj": ("latent", [_p, _ll, _i, _p, _p, _ll, _i, _i, _i, _i, _i, _i, _p]),
     "arle_head_proj_mfma": ("latent", [_p, _ll, _i, _p, _p, _ll, _i, _i, _i, _i, _i, _p]),
-    "arle_moe_route": ("moe", [_p, _ll, _i, _p, _i, _p, _i, _p, _p, _i, _i, _i, _i, _f, _p]),
+    "arle_moe_route": ("moe", [_p, _ll, _i, _p, _i, _p, _i, _p, _p, _i, _i, _i, _i, _f, _i, _i, _i, _i, _p]),
+    "arle_moe_identity": ("moe", [_p, _ll, _i, _p, _p, _i, _i, _i, _i, _p]),
     "arle_moe_expert": ("moe", [_p, _ll, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p]),
+    "arle_gate_mul": ("elementwise", [_p, _ll, _p, _ll, _p, _i, _i, _i, _i, _p]),
+    "arle_token_gate": ("elementwise", [_p, _ll, _i, _p, _ll, _i, _i, _p, _p, _i, _i, _i, _p]),
     "arle_act_mul": ("elementwise", [_p, _p, _ll, _p, _i, _i, _i, _i, _i, _p]),
     "arle_hyper_step": ("hyper", [_p, _ll, _ll, _p, _p, _i, _ll, _i, _ll, _p, _p, _p, _p, _f, _p, _p, _i, _ll, _i, _i, _i,
                                   _i, _p]),
     "arle_pair_norm": ("hyper", [_p, _ll, _i, _ll, _p, _ll, _i, _ll, _i, _p, _p, _f, _f, _p, _i, _i, _i, _p]),
     "arle_rotary_qkv_store": ("rotary_store", [_p, _ll, _p, _ll, _p, _ll, _i, _p, _p, _i, _f, _i, _p, _p, _i, _i, _p, _p,
                                                _p, _i, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
-    "arle_gated_delta_scan": ("gated_delta", [_p, _ll, _p, _ll, _p, _ll, _i, _p, _ll, _p, _p, _f, _p, _p, _p, _i, _i, _p,
-                                              _i, _i, _i, _i, _p]),
-    "arle_gated_delta_output": ("gated_delta", [_p, _p, _ll, _i, _p, _i, _f, _p, _i, _i, _i, _p]),
+    "arle_gated_delta_scan": ("gated_delta", [_p, _ll, _p, _ll, _p, _ll, _i, _p, _ll, _p, _ll, _p, _p, _f, _p, _p, _p, _i, _i, _p,
+                                              _i, _i, _i, _i, _i, _p]),
+    "arle_gated_delta_output": ("gated_delta", [_p, _p, _ll, _i, _p, _i, _f, _p, _i, _i, _i, _i, _p]),
     "arle_ceiling_read": ("ceilings", [_p, _ll, _i, _p, _p, _p]),
     "arle_ceiling_mfma": ("ceilings", [_i, _i, _i, _i, _p, _p]),
 }

@@ -1409,15 +1409,21 @@ LAYERNORM_MAX_WIDTH = 16384
 
 
 def add_layernorm(residual: torch.Tensor, terms, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
-                  weight_b: torch.Tensor | None = None, rows: torch.Tensor | None = None):
-    """residual += sum of `terms` (float32, in place unless `rows` is given); then the layer norm without bias of
-    every row (or of the rows named by `rows`), once with `weight` and, if given, once more with `weight_b`.
+                  weight_b: torch.Tensor | None = None, rows: torch.Tensor | None = None, *,
+                  bias: torch.Tensor | None = None, bias_b: torch.Tensor | None = None):
+    """residual += sum of `terms` (float32, in place unless `rows` is given); then the layer norm of
+    every row (or of the rows named by `rows`), once with `weight` and, if given, once more with `weight_b`;
+    `bias`, `bias_b`: the norms' own biases, of their weights' type (None: none).
 
     terms: up to two (tensor, bias or None); a tensor is [T, H] or a float32 stack [S, T, H] added in order.
     Returns out, or (out, out_b)."""
     terms = list(terms or [])
     _need(len(terms) <= 2, "add_layernorm adds at most two terms")
-    _gpu(residual, weight, weight_b, rows, *[t for pair in terms for t in pair])
+    _gpu(residual, weight, weight_b, rows, bias, bias_b, *[t for pair in terms for t in pair])
+    for c in (bias, bias_b):
+        _need(c is None or (c.shape == weight.shape and c.is_contiguous() and c.dtype == weight.dtype),
+              "a norm's bias must be [width] of its weight's type")
+    _need(bias_b is None or weight_b is not None, "a second bias without a second weight")
     _need(residual.dtype == torch.float32 and residual.dim() == 2 and residual.is_contiguous(),
           "residual must be contiguous float32 [T, H]")
     width = residual.shape[1]
@@ -1436,7 +1442,8 @@ def add_layernorm(residual: torch.Tensor, terms, weight: torch.Tensor, eps: floa
     for i in range(2):
         args += _term_args(*(terms[i] if i < len(terms) else (None, None)), residual.shape)
     lib.call("arle_add_layernorm", residual.data_ptr(), *args, weight.data_ptr(), _ptr(weight_b), _code(weight),
-             out.data_ptr(), _ptr(out_b), _code(out), _ptr(rows), n_rows, width, float(eps), _stream())
+             out.data_ptr(), _ptr(out_b), _code(out), _ptr(rows), n_rows, width, float(eps), _ptr(bias), _ptr(bias_b),
+             _stream())
     return out if weight_b is None else (out, out_b)
 
 
@@ -1619,11 +1626,13 @@ def qkv_norm_store(q, k, v, *, num_q_heads: int, num_kv_heads: int, key_dim: int
 
 def attn_softcap_simt(q, out, k_pages, v_pages, block_table, positions, slot_of_token, *, num_q_heads: int,
                       num_kv_heads: int, key_dim: int, value_dim: int, page_size: int, scale: float,
-                      softcap: float = 0.0, r1=None, r2=None, window: int = 0, chunk: int = 0, sink=None):
+                      softcap: float = 0.0, r1=None, r2=None, window: int = 0, chunk: int = 0, sink=None,
+                      keep_first: int = 0):
     """Causal attention of every row over its request's pages: scores scale (q . k), soft-capped (softcap > 0), less
     r1_h ln(1 + r2_h distance) (r1, r2 [heads] given), over the last `window` keys (0: all) and, with `chunk` > 0,
     over the keys of the row's own chunk of so many positions only; `sink` [heads]: exp(sink_h) joins the softmax's
-    denominator."""
+    denominator; `keep_first` (with a window): the request's first so many keys stay visible behind the window."""
+    _need(keep_first >= 0 and (keep_first == 0 or window > 0), "kept first keys go with a window")
     _gpu(q, out, k_pages, v_pages, block_table, positions, slot_of_token, r1, r2, sink)
     _check_sink(sink, num_q_heads, window, chunk)
     tokens = q.shape[0]
@@ -1646,7 +1655,7 @@ def attn_softcap_simt(q, out, k_pages, v_pages, block_table, positions, slot_of_
              v_pages.data_ptr(), _code(q), block_table.data_ptr(), block_table.shape[1], positions.data_ptr(),
              slot_of_token.data_ptr(), tokens, num_q_heads, num_kv_heads, key_dim, value_dim, page_size, float(scale),
              float(softcap), _ptr(r1), _ptr(r2), _code(r1) if r1 is not None else 0, int(window), int(chunk), _ptr(sink),
-             _code(sink) if sink is not None else 0, _stream())
+             _code(sink) if sink is not None else 0, int(keep_first), _stream())
     return out
 
 
@@ -1671,12 +1680,17 @@ def attn_softcap_mfma_supported(dtype, key_dim: int, value_dim: int, page_size: 
             and key_dim <= CAP_MFMA_MAX_DIM and value_dim <= CAP_MFMA_MAX_DIM)
 
 
-def attn_softcap_mfma_fits(window: int, table_width: int, page_size: int) -> bool:
-    """Whether the ids of the pages that a row's keys span (its window, or all that the block table maps) fit where
-    the matrix-core kernel keeps them."""
+def _softcap_page_ids(window: int, table_width: int, page_size: int, keep_first: int = 0) -> int:
+    """Page ids that a work item of the matrix-core kernel keeps in LDS (the launcher's own count)."""
     mapped = table_width * page_size
     seen = (window + 16 if 0 < window and window + 16 < mapped else mapped) + 64
-    return (seen // page_size + 2) * 4 <= 48 * 1024
+    return seen // page_size + 2 + (keep_first + 31) // page_size + 2
+
+
+def attn_softcap_mfma_fits(window: int, table_width: int, page_size: int, keep_first: int = 0) -> bool:
+    """Whether the ids of the pages that a row's keys span (its window, or all that the block table maps, and the
+    kept first keys) fit where the matrix-core kernel keeps them."""
+    return _softcap_page_ids(window, table_width, page_size, keep_first) * 4 <= 48 * 1024
 
 
 @functools.lru_cache(maxsize=None)
@@ -1686,9 +1700,13 @@ def _softcap_lds_limit() -> int:
 
 def attn_softcap_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, seg_start, *, max_qlen: int,
                       num_q_heads: int, num_kv_heads: int, key_dim: int, value_dim: int, page_size: int, scale: float,
-                      softcap: float = 0.0, r1=None, r2=None, window: int = 0, chunk: int = 0, sink=None):
+                      softcap: float = 0.0, r1=None, r2=None, window: int = 0, chunk: int = 0, sink=None,
+                      keep_first: int = 0):
     """`attn_softcap_simt` on the matrix cores, bfloat16: sixteen rows of a segment a wave, or (when every segment is
-    one decoded row) one row's q heads of a kv head, sixteen at a time, a wave."""
+    one decoded row) one row's q heads of a kv head, sixteen at a time, a wave.  keep_first (with a window and no
+    chunks): the request's first so many keys stay visible to rows whose window has passed them."""
+    _need(keep_first >= 0 and (keep_first == 0 or (window > 0 and chunk == 0)),
+          "kept first keys go with a window and without chunks in the matrix-core kernel")
     _gpu(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot, seg_start, r1, r2, sink)
     _check_sink(sink, num_q_heads, window, chunk)
     tokens = q.shape[0]
@@ -1712,12 +1730,10 @@ def attn_softcap_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot,
     if r1 is not None:
         _need(r1.shape == (num_q_heads,) and r2.shape == (num_q_heads,) and r1.dtype == r2.dtype and r1.dtype in _CODES
               and r1.is_contiguous() and r2.is_contiguous(), "r1, r2 must be [heads] of one type")
-    _need(attn_softcap_mfma_fits(mask_span(window, chunk), block_table.shape[1], page_size),
+    _need(attn_softcap_mfma_fits(mask_span(window, chunk), block_table.shape[1], page_size, keep_first),
           "the keys a row sees span more pages than the kernel holds ids for")
     # a decoded row's waves add their sums through LDS: that and the page ids have to fit a compute unit's
-    mapped = block_table.shape[1] * page_size
-    span = mask_span(window, chunk)
-    page_ids = ((span + 16 if 0 < span and span + 16 < mapped else mapped) + 64) // page_size + 2
+    page_ids = _softcap_page_ids(mask_span(window, chunk), block_table.shape[1], page_size, keep_first)
     heads_mode = (max_qlen == 1 and segments == tokens
                   and 8 * ((value_dim // 16) * 256 + 32) * 4 + page_ids * 4 <= _softcap_lds_limit())
     row_blocks = tokens // 16 + segments      # no fewer than the sixteen-row blocks of all segments together
@@ -1726,16 +1742,26 @@ def attn_softcap_mfma(q, out, k_pages, v_pages, block_table, seg_row0, seg_slot,
              seg_start.data_ptr(), segments, row_blocks, 1 if heads_mode else 0, num_q_heads, num_kv_heads, key_dim,
              value_dim, page_size, float(scale), float(softcap), _ptr(r1), _ptr(r2),
              _code(r1) if r1 is not None else 0, int(window), int(chunk), _ptr(sink),
-             _code(sink) if sink is not None else 0, _stream())
+             _code(sink) if sink is not None else 0, int(keep_first), _stream())
     return out
 
 
 def wide_norm_store(q, k, v, *, num_q_heads: int, num_kv_heads: int, key_dim: int, value_dim: int, eps: float,
                     q_weight=None, k_weight=None, v_first=None, mix=None, positions, slot_of_token, block_table,
-                    k_pages, v_pages, page_size: int):
+                    k_pages, v_pages, page_size: int, cos=None, sin=None, rotary_dim: int = 0, interleaved: bool = False):
     """RMS norm of q over its whole row (in place, weight [heads * Dk]) and of k over its whole row (weight
     [kv heads * Dk]); k goes to the pages, and so does v, as (1 - mix) v + mix v_first where v_first [T, kv heads * Dv]
-    is given (`mix`: a tensor of one number)."""
+    is given (`mix`: a tensor of one number).  rotary_dim > 0: behind the norm the first so many entries of every head
+    of q and k turn by the angles of the float32 tables cos, sin [positions, rotary_dim / 2] (entry i with
+    i + rotary_dim / 2, or with `interleaved` 2i with 2i + 1)."""
+    _need(0 <= rotary_dim <= key_dim and rotary_dim % 2 == 0, "rotary_dim must be even and at most the head's size")
+    _need(max(num_q_heads, num_kv_heads) * key_dim * 4 <= 64 * 1024 or not rotary_dim,
+          "a rotated row of more than 16,384 entries is not taken")
+    if rotary_dim:
+        _gpu(cos, sin)
+        for name, t in (("cos", cos), ("sin", sin)):
+            _need(t is not None and t.dtype == torch.float32 and t.dim() == 2 and t.shape[1] == rotary_dim // 2
+                  and t.is_contiguous(), f"{name} must be contiguous float32 [positions, rotary_dim / 2]")
     _gpu(q, k, v, q_weight, k_weight, v_first, mix, positions, slot_of_token, block_table, k_pages, v_pages)
     tokens = q.shape[0]
     for name, t, width in (("q", q, num_q_heads * key_dim), ("k", k, num_kv_heads * key_dim),
@@ -1763,7 +1789,8 @@ def wide_norm_store(q, k, v, *, num_q_heads: int, num_kv_heads: int, key_dim: in
              w_code, _ptr(mix) if v_first is not None else 0, _code(mix) if v_first is not None else 0, float(eps),
              positions.data_ptr(), slot_of_token.data_ptr(), block_table.data_ptr(), block_table.shape[1],
              k_pages.data_ptr(), v_pages.data_ptr(), tokens, num_q_heads, num_kv_heads, key_dim, value_dim,
-             int(page_size), _stream())
+             int(page_size), _ptr(cos) if rotary_dim else 0, _ptr(sin) if rotary_dim else 0, int(rotary_dim),
+             0 if interleaved else 1, _stream())
 
 
 # ------------------------------------------------------------------ a norm on a sublayer's output
@@ -1790,9 +1817,11 @@ def _addend_args(term, rows: int, width: int):
 
 
 def norm_add(residual: torch.Tensor, terms, weight: torch.Tensor, eps: float, *, one_plus: bool = False,
-             act_dtype: torch.dtype | None = None):
-    """residual += y / sqrt(mean(y^2) + eps) * weight (or 1 + weight) for y the sum of up to two `terms`, in place;
-    returns the updated residual rounded to `act_dtype` (None: nothing is returned)."""
+             act_dtype: torch.dtype | None = None, center: bool = False, bias: torch.Tensor | None = None,
+             mult: float = 1.0):
+    """residual += mult * y / sqrt(mean(y^2) + eps) * weight (or 1 + weight) for y the sum of up to two `terms`, in
+    place; with `center` the layer norm mult * ((y - mean) / sqrt(var + eps) * weight + bias) instead (bias [width] of
+    the weight's type, or None); returns the updated residual rounded to `act_dtype` (None: nothing is returned)."""
     terms = [t for t in (terms if isinstance(terms, list) else [terms]) if t is not None]
     _need(1 <= len(terms) <= 2, "norm_add takes one or two addends")
     # what a sublayer leaves for the residual is 32-bit sums; an output that was rounded on its way is widened first
@@ -1803,12 +1832,14 @@ def norm_add(residual: torch.Tensor, terms, weight: torch.Tensor, eps: float, *,
     rows, width = residual.shape
     _need(0 < width <= NORM_ADD_MAX_WIDTH, f"norm_add takes widths up to {NORM_ADD_MAX_WIDTH}")
     _need(weight.shape == (width,) and weight.is_contiguous() and weight.dtype in _CODES, "norm weight must be [width]")
+    _need(bias is None or (bias.is_cuda and bias.shape == (width,) and bias.is_contiguous() and bias.dtype == weight.dtype),
+          "a norm's bias must be [width] of its weight's type")
     act = torch.empty((rows, width), dtype=act_dtype, device=residual.device) if act_dtype is not None else None
     args = []
     for i in range(2):
         args += _addend_args(terms[i] if i < len(terms) else None, rows, width)
     lib.call("arle_norm_add", residual.data_ptr(), *args, weight.data_ptr(), _code(weight), 1 if one_plus else 0,
-             _ptr(act), _code(act) if act is not None else 0, rows, width, float(eps), _stream())
+             1 if center else 0, _ptr(bias), float(mult), _ptr(act), _code(act) if act is not None else 0, rows, width, float(eps), _stream())
     return act
 
 
@@ -1826,9 +1857,10 @@ HEAD_PROJ_MAX_K = 1024
 
 
 def latent_prep(q, dkv, q_full, *, heads: int, dim: int, rot_dim: int, rank: int, c_weight, eps: float, cos, sin,
-                rotary_dims: int, positions, slot_of_token, block_table, k_pages, v_pages, page_size: int):
+                rotary_dims: int, positions, slot_of_token, block_table, k_pages, v_pages, page_size: int,
+                halves: bool = False):
     """dkv [T, rank + rot_dim]: the first `rank` entries RMS-normed (c), the rest rotated (interleaved pairs over the
-    first `rotary_dims`), [c | k_rot] to the key pages and c to the value pages; the rotated part of every head of
+    first `rotary_dims`, or with `halves` entry i with i + rotary_dims / 2), [c | k_rot] to the key pages and c to the value pages; the rotated part of every head of
     q [T, heads * (dim + rot_dim)] goes, rotated, to the last rot_dim entries of its head in
     q_full [T, heads * (rank + rot_dim)]."""
     _gpu(q, dkv, q_full, c_weight, cos, sin, positions, slot_of_token, block_table, k_pages, v_pages)
@@ -1852,7 +1884,7 @@ def latent_prep(q, dkv, q_full, *, heads: int, dim: int, rot_dim: int, rank: int
              q_full.stride(0), _code(q), c_weight.data_ptr(), _code(c_weight), float(eps), _ptr(cos), _ptr(sin),
              int(rotary_dims), positions.data_ptr(), slot_of_token.data_ptr(), block_table.data_ptr(),
              block_table.shape[1], k_pages.data_ptr(), v_pages.data_ptr(), tokens, heads, dim, rot_dim, rank,
-             int(page_size), _stream())
+             int(page_size), 1 if halves else 0, _stream())
 
 
 def head_proj(x, wt, out, *, heads: int, in_head: int, out_head: int):
@@ -1900,10 +1932,14 @@ MOE_MAX_EXPERTS = 1024
 MOE_MAX_TOP = 64
 
 
-def moe_route(x, router, correction, *, top: int, scale: float):
-    """(ids int32 [T, top], weights float32 [T, top]) of a sigmoid router: z = router x in 32-bit sums,
-    s = sigmoid(z), the `top` largest s + correction chosen (ties: the lower index), weights s / (sum + 1e-20) * scale
-    in the order they were chosen."""
+def moe_route(x, router, correction, *, top: int, scale: float, score: str = "sigmoid", groups: int = 1,
+              keep_groups: int = 1, normalize: bool = True):
+    """(ids int32 [T, top], weights float32 [T, top]) of a router: z = router x in 32-bit sums, s = sigmoid(z) or
+    (score "softmax") softmax(z) over all rows of the router, the `top` largest s + correction chosen (ties: the lower
+    index) among the experts of the `keep_groups` best of `groups` equal groups of neighbours (a group's number: the
+    largest s + correction in it), weights s / (sum + 1e-20) * scale, or s * scale without `normalize`, in the order
+    they were chosen."""
+    _need(score in ("sigmoid", "softmax"), "a router's scores are sigmoid or softmax")
     _gpu(x, router, correction)
     _rows(x, "x")
     experts, width = router.shape
@@ -1911,6 +1947,8 @@ def moe_route(x, router, correction, *, top: int, scale: float):
           "router must be contiguous [experts, width]")
     _need(1 <= top <= min(experts, MOE_MAX_TOP) and experts <= MOE_MAX_EXPERTS,
           f"the router takes up to {MOE_MAX_EXPERTS} experts and {MOE_MAX_TOP} choices a token")
+    _need(groups >= 1 and experts % groups == 0 and 1 <= keep_groups <= groups and top <= keep_groups * (experts // groups),
+          "groups divide the experts evenly, and the kept groups hold at least `top` experts")
     if correction is not None:
         _need(correction.shape == (experts,) and correction.is_contiguous() and correction.dtype in _CODES,
               "correction must be [experts]")
@@ -1918,8 +1956,24 @@ def moe_route(x, router, correction, *, top: int, scale: float):
     weights = torch.empty((x.shape[0], top), dtype=torch.float32, device=x.device)
     lib.call("arle_moe_route", x.data_ptr(), x.stride(0), _code(x), router.data_ptr(), _code(router), _ptr(correction),
              _code(correction) if correction is not None else 0, ids.data_ptr(), weights.data_ptr(), x.shape[0], width,
-             experts, int(top), float(scale), _stream())
+             experts, int(top), float(scale), 1 if score == "softmax" else 0, int(groups), int(keep_groups),
+             1 if normalize else 0, _stream())
     return ids, weights
+
+
+def moe_identity(x, ids, outs, first: int):
+    """Rows of experts that hand back their input: where ids [T, top] names a router output from `first` on, the row
+    t * top + k of outs (float32 [T * top, W]) becomes x[t] (in 32 bits)."""
+    _gpu(x, ids, outs)
+    _rows(x, "x")
+    tokens, top = ids.shape
+    _need(ids.dtype == torch.int32 and ids.is_contiguous() and x.shape[0] == tokens and x.dtype in _CODES,
+          "ids must be contiguous int32 [T, top] over the rows of x")
+    _need(outs.dtype == torch.float32 and outs.is_contiguous() and outs.shape == (tokens * top, x.shape[1]),
+          "outs must be contiguous float32 [T * top, W]")
+    lib.call("arle_moe_identity", x.data_ptr(), x.stride(0), _code(x), ids.data_ptr(), outs.data_ptr(), tokens, top,
+             x.shape[1], int(first), _stream())
+    return outs
 
 
 def moe_expert(x, w, ids, *, gate_up: bool):
@@ -1943,8 +1997,40 @@ def moe_expert(x, w, ids, *, gate_up: bool):
 
 # ------------------------------------------------------------- gated feed-forward activations
 
-ACT_SILU, ACT_GELU_TANH = 0, 1
-ACTIVATIONS = {"silu": ACT_SILU, "gelu_tanh": ACT_GELU_TANH}
+ACT_SILU, ACT_GELU_TANH, ACT_SIGMOID = 0, 1, 2
+ACTIVATIONS = {"silu": ACT_SILU, "gelu_tanh": ACT_GELU_TANH}      # of a gated feed-forward's gate
+GATES = dict(ACTIVATIONS, sigmoid=ACT_SIGMOID)                    # of a gate on something that is not its own input
+
+
+def gate_mul(gate: torch.Tensor, x: torch.Tensor, act: int = ACT_SIGMOID):
+    """out = act(gate) * x for two [T, W] views of one type, each with a row stride of its own; out is contiguous."""
+    _gpu(gate, x)
+    _rows(gate, "gate")
+    _rows(x, "x")
+    _need(gate.shape == x.shape and gate.dtype == x.dtype and gate.dtype in _CODES, "gate and x must agree in shape and type")
+    _need(act in GATES.values(), "unknown activation code")
+    tokens, width = gate.shape
+    _need(math.ceil(width / 256) <= _GRID_Y_MAX, "gate_mul: width too large")
+    out = torch.empty((tokens, width), dtype=gate.dtype, device=gate.device)
+    lib.call("arle_gate_mul", gate.data_ptr(), gate.stride(0), x.data_ptr(), x.stride(0), out.data_ptr(), _code(gate),
+             tokens, width, int(act), _stream())
+    return out
+
+
+def token_gate(z: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, first: int, act: int = ACT_GELU_TANH):
+    """out[t, j] = act(z[t, j]) * table[ids[t], first + j]: z [T, W], table [rows, >= first + W] (bfloat16 or float32),
+    ids int32 [T] inside the table (the step's token ids, which the engine has checked against the vocabulary)."""
+    _gpu(z, table, ids)
+    _rows(z, "z")
+    tokens, width = z.shape
+    _need(z.dtype in _CODES and table.dtype in _CODES and table.dim() == 2 and table.stride(1) == 1, "table must be [rows, columns]")
+    _need(0 <= first and first + width <= table.shape[1], "the slice does not lie in the table's columns")
+    _i32(ids, "ids", tokens)
+    _need(act in GATES.values(), "unknown activation code")
+    out = torch.empty((tokens, width), dtype=z.dtype, device=z.device)
+    lib.call("arle_token_gate", z.data_ptr(), z.stride(0), _code(z), table.data_ptr(), table.stride(0), _code(table),
+             int(first), ids.data_ptr(), out.data_ptr(), tokens, width, int(act), _stream())
+    return out
 
 
 def act_mul(gate: torch.Tensor, up: torch.Tensor, act: int = ACT_SILU):
@@ -2104,12 +2190,14 @@ GATED_DELTA_MAX_KEY_DIM = 256
 
 
 def gated_delta_scan(q, k, v, gates, a_log, dt_bias, s_state, seg_row0, seg_slot, *, heads: int, kv_heads: int,
-                     key_dim: int, value_dim: int, unit_eps: float = 1e-6):
+                     key_dim: int, value_dim: int, unit_eps: float = 1e-6, channel_decay=None):
     """The gated delta rule over the rows of every segment, from and into the requests' states (see
     csrc/gated_delta.hip).  q, k [T, kv_heads * D] and v [T, heads * Dv] as the convolutions left them; gates float32
     [T, >= 2 * heads]: the pre-activations of beta, then those of the decay; a_log, dt_bias float32 [heads]; s_state
-    float32 [slots, heads, D, Dv].  Returns o float32 [T, heads * Dv]."""
-    _gpu(q, k, v, gates, a_log, dt_bias, s_state, seg_row0, seg_slot)
+    float32 [slots, heads, D, Dv].  channel_decay: float32 [T, heads * D], the pre-activations of a decay for every
+    head and key entry; gates then holds beta's alone ([T, >= heads]) and dt_bias is [heads * D].
+    Returns o float32 [T, heads * Dv]."""
+    _gpu(q, k, v, gates, a_log, dt_bias, s_state, seg_row0, seg_slot, channel_decay)
     H, G, D, Dv = heads, kv_heads, key_dim, value_dim
     tokens = q.shape[0]
     for name, t, width in (("q", q, G * D), ("k", k, G * D), ("v", v, H * Dv)):
@@ -2118,25 +2206,35 @@ def gated_delta_scan(q, k, v, gates, a_log, dt_bias, s_state, seg_row0, seg_slot
     _need(0 < D <= GATED_DELTA_MAX_KEY_DIM and G > 0 and H % G == 0 and H <= _GRID_Y_MAX,
           f"key sizes up to {GATED_DELTA_MAX_KEY_DIM}, heads a multiple of the q/k heads")
     _rows(gates, "gates")
-    _need(gates.dtype == torch.float32 and gates.shape[0] == tokens and gates.shape[1] >= 2 * H, "gates must be float32 [T, >= 2 * heads]")
-    _need(a_log.shape == (H,) and dt_bias.shape == (H,) and a_log.dtype == dt_bias.dtype == torch.float32
-          and a_log.is_contiguous() and dt_bias.is_contiguous(), "A_log and dt_bias must be float32 [heads]")
+    channel = channel_decay is not None
+    _need(gates.dtype == torch.float32 and gates.shape[0] == tokens and gates.shape[1] >= (H if channel else 2 * H),
+          "gates must be float32 [T, >= 2 * heads] (with a decay a channel: [T, >= heads])")
+    decays = H * D if channel else H
+    if channel:
+        _rows(channel_decay, "channel_decay")
+        _need(channel_decay.dtype == torch.float32 and channel_decay.shape == (tokens, decays),
+              "the channels' decays must be float32 [T, heads * D]")
+    _need(a_log.shape == (H,) and dt_bias.shape == (decays,) and a_log.dtype == dt_bias.dtype == torch.float32
+          and a_log.is_contiguous() and dt_bias.is_contiguous(), "A_log must be float32 [heads], dt_bias float32 [decays]")
     _need(s_state.dim() == 4 and tuple(s_state.shape[1:]) == (H, D, Dv) and s_state.dtype == torch.float32
           and s_state.is_contiguous(), "the state is float32 [slots, heads, D, Dv]")
     segments = seg_slot.numel()
     _i32(seg_slot, "seg_slot")
     _i32(seg_row0, "seg_row0", segments + 1)
     out = torch.empty((tokens, H * Dv), dtype=torch.float32, device=q.device)
+    decay_ptr = channel_decay.data_ptr() if channel else gates.data_ptr() + 4 * H
+    decay_stride = channel_decay.stride(0) if channel else gates.stride(0)
     lib.call("arle_gated_delta_scan", q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0),
-             _code(q), gates.data_ptr(), gates.stride(0), a_log.data_ptr(), dt_bias.data_ptr(), float(unit_eps),
-             s_state.data_ptr(), seg_row0.data_ptr(), seg_slot.data_ptr(), segments, 1 if tokens == segments else 0,
-             out.data_ptr(), H, G, D, Dv, _stream())
+             _code(q), gates.data_ptr(), gates.stride(0), decay_ptr, decay_stride, a_log.data_ptr(), dt_bias.data_ptr(),
+             float(unit_eps), s_state.data_ptr(), seg_row0.data_ptr(), seg_slot.data_ptr(), segments,
+             1 if tokens == segments else 0, out.data_ptr(), H, G, D, Dv, 1 if channel else 0, _stream())
     return out
 
 
-def gated_delta_output(o, gate, weight, eps: float, *, heads: int, value_dim: int):
-    """Each head's o [T, heads * Dv] (float32) divided by its root mean square, times weight [Dv], times silu(gate);
-    in the type of `gate`."""
+def gated_delta_output(o, gate, weight, eps: float, *, heads: int, value_dim: int, act: int = 0):
+    """Each head's o [T, heads * Dv] (float32) divided by its root mean square, times weight [Dv], times act(gate)
+    (act 0: silu; one of GATES' codes); in the type of `gate`."""
+    _need(act in (0, 1, 2), "unknown activation code")
     _gpu(o, gate, weight)
     tokens = o.shape[0]
     width = heads * value_dim
@@ -2147,5 +2245,5 @@ def gated_delta_output(o, gate, weight, eps: float, *, heads: int, value_dim: in
     _need(heads <= _GRID_Y_MAX, "too many heads")
     out = torch.empty((tokens, width), dtype=gate.dtype, device=o.device)
     lib.call("arle_gated_delta_output", o.data_ptr(), gate.data_ptr(), gate.stride(0), _code(gate), weight.data_ptr(),
-             _code(weight), float(eps), out.data_ptr(), tokens, heads, value_dim, _stream())
+             _code(weight), float(eps), out.data_ptr(), tokens, heads, value_dim, int(act), _stream())
     return out

@@ -1,5 +1,5 @@
 """Architectures known to the registry.  Importing this package registers them."""
-from . import gufasun, qwen3, sovutar, tazitar  # noqa: F401
+from . import gufasun, qwen3, retudra, sovutar, tazitar  # noqa: F401
 from .decoder import (DecoderModel, build_model, declared_cache_needs, expected_checkpoint_tensors,
                       kv_cache_bytes_per_token)
 

@@ -14,7 +14,7 @@ from ..kernels import ops
 from ..parts import base  # noqa: F401  (registries)
 from ..parts import (attention, block, embedding, feed_forward, gated_delta, hyper, latent_attention,  # noqa: F401  registers the stock parts
                      mixer_pair, mlstm, moe, norm, position, rotary_attention, short_conv, softcap_attention,
-                     wide_norm_attention)
+                     token_side, wide_norm_attention)
 from ..parts.base import Runtime, build_part, expected_tensors, lookup
 from ..parts.spec import ModelSpec
 

@@ -36,20 +36,28 @@ class PreNormBlock:
 @register("block", "post_norm")
 class PostNormBlock:
     """h += norm_a(mixer(h)); h += norm_b(ffn(h)): the sublayers read the residual itself, the norms stand on their
-    outputs.  norm roles: "mixer_out", "ffn_out" (the second only with a feed-forward).  The residual is float32;
+    outputs (a norm's `add_scale` is the model's factor on what is added).  norm roles: "mixer_out", "ffn_out" (the
+    second only with a feed-forward), "side_out" (with a further part "side").  The residual is float32;
     what a sublayer reads is the residual in the activation type, which the norm's kernel writes beside the sum it
     updates (`add_into`), and which goes from block to block in `batch.carry`.  Nothing is left for the next block
-    to add."""
+    to add.
 
-    norm_roles = ("mixer_out", "ffn_out")
+    A further part named "side" (a feed-forward that also reads the step's tokens: `forward(x, batch)`) runs behind
+    the feed-forward as a third sublayer of the same kind: h += norm_c(side(h, tokens))."""
+
+    norm_roles = ("mixer_out", "ffn_out", "side_out")
     CARRY = "residual_rounded"     # batch.carry[CARRY] = (the residual tensor, its copy in the activation type)
 
-    def __init__(self, mixer, feed_forward, norms: dict):
+    def __init__(self, mixer, feed_forward, norms: dict, extra: dict | None = None):
         self.mixer = mixer
         self.feed_forward = feed_forward
         self.norms = norms
         self.norm_mixer = norms.get("mixer_out") if mixer is not None else None
         self.norm_ffn = norms.get("ffn_out") if feed_forward is not None else None
+        self.side = (extra or {}).get("side")
+        self.norm_side = norms.get("side_out") if self.side is not None else None
+        if self.side is not None and self.norm_side is None:
+            raise ValueError("a post_norm block with a side part needs the norm on its output (side_out)")
 
     def _reads(self, residual, batch):
         kept = batch.carry.get(self.CARRY)
@@ -69,6 +77,8 @@ class PostNormBlock:
             x = self.norm_mixer.add_into(residual, self.mixer.forward(x, batch, cache_view))
         if self.feed_forward is not None:
             x = self.norm_ffn.add_into(residual, self.feed_forward.forward(x))
+        if self.side is not None:
+            x = self.norm_side.add_into(residual, self.side.forward(x, batch))
         batch.carry[self.CARRY] = (residual, x)
         return residual, None
 

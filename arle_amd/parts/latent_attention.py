@@ -8,14 +8,14 @@ latent size C:
     k_h = W_uk,h c,  v_h = W_uv,h c
     s_ij,h = scale (q_h,i . k_h,j + rotate(q_rot,h,i) . k_rot,j)    for 0 <= i - j < window  (None: every j <= i)
     p = exp(s) / (sum_j exp(s_ij) + exp(sink_h))            (sink: a learned number a head, optional)
-    out = W_o concat_h(sum_j p_j v_h,j)
+    out = W_o (concat_h(sum_j p_j v_h,j) * sigmoid(W_g h))          (the gate: optional)
 
 The maps W_uk and W_uv are folded into the query and the output: q'_h = W_uk,h^T q_h, so that
 s = scale (q'_h . c + q_rot . k_rot), and out_h = W_uv,h (sum_j p_j c_j).  The attention is then one of H query heads
 over a single key/value head with keys [c | k_rot] and values c, which is what the pages hold
 (`[1, page, C + R]`, and c once more d-major `[1, C, page]` as the second operand of the matrix cores); keys and
-values of the heads are never formed.  The rotation is a position part (`rope_interleaved`) whose table the
-preparation kernel reads.
+values of the heads are never formed.  The rotation is a position part (`rope_interleaved`, pairs (2i, 2i + 1), or
+`rope_neox`, pairs (i, i + R'/2) over the first R' rotated entries) whose table the preparation kernel reads.
 """
 from __future__ import annotations
 
@@ -31,7 +31,8 @@ from .softcap_attention import softcap_attention
 @register("mixer", "latent_attention")
 class LatentAttention(Part):
     """params: hidden_size, heads, dim, rot_dim, value_dim, rank, eps, scale, window (int | None), sink (bool),
-    position (PartSpec of the rotation over the rot_dim part)."""
+    gate (bool: a sigmoid gate on the heads' outputs, a projection of the mixer's input), position (PartSpec of the
+    rotation over the rot_dim part)."""
 
     graph_safe = True  # positions, slots and lengths are read on the GPU; launches depend on shapes only
 
@@ -43,6 +44,8 @@ class LatentAttention(Part):
                 "uk": WeightDecl((H * D, C)), "uv": WeightDecl((H * Dv, C)), "o": WeightDecl((h, H * Dv))}
         if params.get("sink"):
             decl["sink"] = WeightDecl((H,), init="normal")
+        if params.get("gate"):
+            decl["g"] = WeightDecl((H * Dv, h))
         return decl
 
     @classmethod
@@ -72,10 +75,13 @@ class LatentAttention(Part):
         self.window = int(params.get("window") or 0)
         self.position = children["position"]
         wq, wd = tensors["q"], tensors["dkv"]
-        if len({wq.dtype, wd.dtype, tensors["uk"].dtype, tensors["uv"].dtype}) != 1:
+        self.gated = bool(params.get("gate"))
+        fused = [wq, wd] + ([tensors["g"]] if self.gated else [])
+        if len({t.dtype for t in fused} | {tensors["uk"].dtype, tensors["uv"].dtype}) != 1:
             raise ValueError("the projections of a latent attention must be stored in one type")
         self.q_width = self.H * (self.D + self.R)
-        self.proj = Linear(torch.cat([wq, wd], dim=0).contiguous(), rt.weight_tiles)
+        self.dkv_width = self.C + self.R
+        self.proj = Linear(torch.cat(fused, dim=0).contiguous(), rt.weight_tiles)
         self.c_norm = tensors["c_norm"]
         # a matrix a head, stored [inner, outer]: q'_h = q_h W_uk,h (W_uk,h is [D, C] as it lies), out_h = lat_h W_uv,h^T
         # (the matrix-core form of the product reads the other layout, [outer, inner]; only the one that runs is kept)
@@ -92,7 +98,7 @@ class LatentAttention(Part):
     def products(self):
         if self.proj.weight.dtype != torch.bfloat16:
             return []
-        return [("q_dkv", self.proj.out_features, self.proj.in_features, False, None),
+        return [("q_dkv_g" if self.gated else "q_dkv", self.proj.out_features, self.proj.in_features, False, None),
                 ("o", self.o.out_features, self.o.in_features, False, "norm")]
 
     def _per_head(self, x, which, out, *, in_head, out_head):
@@ -113,16 +119,18 @@ class LatentAttention(Part):
         self.position.ensure_positions(batch.max_position + 1)
         cos, sin, rot = self.position.fused_rotary()
         y = self.proj(x)
-        q, dkv = y[:, :self.q_width], y[:, self.q_width:]
+        q, dkv = y[:, :self.q_width], y[:, self.q_width:self.q_width + self.dkv_width]
         q_full = torch.empty((x.shape[0], H * (C + R)), dtype=x.dtype, device=x.device)
         ops.latent_prep(q, dkv, q_full, heads=H, dim=D, rot_dim=R, rank=C, c_weight=self.c_norm, eps=self.eps, cos=cos,
                         sin=sin, rotary_dims=rot, positions=batch.positions, slot_of_token=batch.slot_of_token,
                         block_table=cache.block_table, k_pages=cache.pages["k"], v_pages=cache.pages["v"],
-                        page_size=cache.page_size)
+                        page_size=cache.page_size, halves=self.position.kind != "rope_interleaved")
         self._per_head(q, "uk", q_full, in_head=D + R, out_head=C + R)
         latent = torch.empty((x.shape[0], H * C), dtype=x.dtype, device=x.device)
         softcap_attention(q_full, latent, cache, batch, num_q_heads=H, num_kv_heads=1, key_dim=C + R, value_dim=C,
                           scale=self.scale, softcap=0.0, r1=None, r2=None, window=self.window, sink=self.sink)
         heads_out = torch.empty((x.shape[0], H * Dv), dtype=x.dtype, device=x.device)
         self._per_head(latent, "uv", heads_out, in_head=C, out_head=Dv)
+        if self.gated:
+            heads_out = ops.gate_mul(y[:, self.q_width + self.dkv_width:], heads_out, ops.ACT_SIGMOID)
         return self.o(heads_out, out_dtype=torch.float32, partials_ok=True)   # into the 32-bit residual unrounded

@@ -151,16 +151,18 @@ class SoftcapAttention(Part):
 
 
 def softcap_attention(q, out, kv, batch, *, num_q_heads, num_kv_heads, key_dim, value_dim, scale, softcap, r1, r2,
-                      window, chunk=0, sink=None):
+                      window, chunk=0, sink=None, keep_first=0):
     """Attention of every row of the packed step over its request's pages: bfloat16 pages of sizes the matrix-core
     kernel takes run there; float32 pages, and every other shape, run the fixed-order kernel (the true 32-bit path).
     chunk > 0: a row sees the keys of its own chunk of so many positions only; sink [heads]: a term exp(sink_h) in the
-    softmax's denominator."""
-    common = dict(num_q_heads=num_q_heads, num_kv_heads=num_kv_heads, key_dim=key_dim, value_dim=value_dim,
+    softmax's denominator; keep_first (with a window): the request's first so many keys stay visible to rows whose
+    window has passed them, at their true positions."""
+    common = dict(keep_first=keep_first, num_q_heads=num_q_heads, num_kv_heads=num_kv_heads, key_dim=key_dim, value_dim=value_dim,
                   page_size=kv.page_size, scale=scale, softcap=softcap, r1=r1, r2=r2, window=window, chunk=chunk, sink=sink)
     if (ops.attn_softcap_mfma_supported(q.dtype, key_dim, value_dim, kv.page_size, num_q_heads // num_kv_heads)
             and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0
-            and ops.attn_softcap_mfma_fits(ops.mask_span(window, chunk), kv.block_table.shape[1], kv.page_size)):
+            and not (keep_first and chunk)
+            and ops.attn_softcap_mfma_fits(ops.mask_span(window, chunk), kv.block_table.shape[1], kv.page_size, keep_first)):
         ops.attn_softcap_mfma(q, out, kv.pages["k"], kv.pages["v"], kv.block_table, batch.seg_row0, batch.seg_slot,
                               batch.seg_start, max_qlen=batch.max_qlen, **common)
     else:

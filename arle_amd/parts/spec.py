@@ -20,7 +20,9 @@ from dataclasses import dataclass, field
 
 @dataclass(frozen=True)
 class WeightDecl:
-    """What a part expects of one parameter: its shape and how random weights fill it."""
+    """What a part expects of one parameter: its shape and how random weights fill it.  A size of None is one that
+    the checkpoint's tensor gives itself (the width of a narrow middle between two projections, say): the loader takes
+    any size there, and the part checks what has to agree."""
 
     shape: tuple
     init: str = "normal"  # a name known to weights.random_init: "normal" N(0, std), "ones" 1 + N(0, norm_std), "zeros", ...

@@ -99,8 +99,10 @@ def compare_with_expected(found: dict, expected: dict, strict: bool = False) -> 
     names the model does not know (never fatal alone unless `strict`)."""
     missing = sorted(n for n in expected if n not in found)
     unexpected = sorted(n for n in found if n not in expected)
+    # (an expected size of None is one that the tensor itself gives: any size fits there)
+    fits = lambda want, have: len(want) == len(have) and all(w is None or w == h for w, h in zip(want, have))
     wrong = sorted((n, tuple(expected[n].shape), tuple(found[n])) for n in expected
-                   if n in found and tuple(found[n]) != tuple(expected[n].shape))
+                   if n in found and not fits(tuple(expected[n].shape), tuple(found[n])))
     if not (missing or wrong or (strict and unexpected)):
         return unexpected
     lines = ["checkpoint does not match the model:"]

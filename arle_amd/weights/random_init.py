@@ -81,6 +81,9 @@ def random_tensor(name: str, decl, seed: int, std: float, norm_std: float, dtype
     except KeyError:
         raise ValueError(f"tensor '{name}': no way to fill a weight of kind {decl.init!r} is registered "
                          f"(known: {', '.join(sorted(INITS))})") from None
+    if any(d is None for d in decl.shape):
+        raise ValueError(f"tensor '{name}': a size that only a checkpoint gives ({list(decl.shape)}) must be named in the "
+                         "configuration before random weights can be made")
     return fill(tuple(decl.shape), gen, std, norm_std, device).to(dtype)
 
 
