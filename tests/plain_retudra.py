@@ -11,9 +11,18 @@ import torch
 
 F = torch.float64
 
+# a test may set this to a function of a matrix product's result (to move every entry by a rounding, say)
+after_product = None
+
 
 def t64(x):
     return x.to(F)
+
+
+def mm(x, w):
+    """x [.., K] times w [N, K] transposed: every projection goes through here."""
+    y = x @ w.T
+    return after_product(y) if after_product is not None else y
 
 
 def gelu_tanh(z):
@@ -69,7 +78,7 @@ def attention(h, m, w, eps):
     """The windowed grouped-query attention.  m: the layer's `mixer` dictionary, w(name) -> tensor of the mixer."""
     T = h.shape[0]
     H, G, D, Dv = m["heads"], m.get("kv_heads") or m["heads"], m["dim"], m["vdim"]
-    q, k, v = h @ w("q").T, h @ w("k").T, h @ w("v").T
+    q, k, v = mm(h, w("q")), mm(h, w("k")), mm(h, w("v"))
     q = rms_norm(q, w("q.norm"), eps).view(T, H, D)           # over all heads' entries at once
     k = rms_norm(k, w("k.norm"), eps).view(T, G, D)
     pos = torch.arange(T)
@@ -82,7 +91,7 @@ def attention(h, m, w, eps):
     mask = m.get("mask")
     see = visible(T, mask["size"], mask.get("keep_first", 0)) if mask else visible(T)
     o = softmax_attention(q, k, v, m["scale"], see)
-    return o.reshape(T, H * Dv) @ w("o").T
+    return mm(o.reshape(T, H * Dv), w("o"))
 
 
 def latent_attention(h, m, w, eps):
@@ -90,21 +99,21 @@ def latent_attention(h, m, w, eps):
     that all heads share and a sigmoid gate on the heads' outputs."""
     T = h.shape[0]
     H, D, R, Dv, C = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
-    q = (h @ w("q").T).view(T, H, D + R)
-    d = h @ w("dkv").T
+    q = mm(h, w("q")).view(T, H, D + R)
+    d = mm(h, w("dkv"))
     c = rms_norm(d[:, :C], w("dkv.norm"), eps)
     k_rot = d[:, C:].view(T, 1, R)
     pos = torch.arange(T)
     rot = m["rot"]
     q_rot = rotate_half(q[..., D:], pos, rot["dims"], rot["base"])
     k_rot = rotate_half(k_rot, pos, rot["dims"], rot["base"]).expand(T, H, R)
-    k_plain = (c @ w("uk").T).view(T, H, D)
-    v = (c @ w("uv").T).view(T, H, Dv)
+    k_plain = mm(c, w("uk")).view(T, H, D)
+    v = mm(c, w("uv")).view(T, H, Dv)
     qq = torch.cat([q[..., :D], q_rot], dim=-1)
     kk = torch.cat([k_plain, k_rot], dim=-1)
     o = softmax_attention(qq, kk, v, m["scale"], visible(T)).reshape(T, H * Dv)
-    o = o * torch.sigmoid(h @ w("g").T)
-    return o @ w("o").T
+    o = o * torch.sigmoid(mm(h, w("g")))
+    return mm(o, w("o"))
 
 
 def causal_conv(x, taps):
@@ -121,15 +130,15 @@ def channel_delta(h, m, w, eps):
     """The gated delta rule with a decay for every head and key channel."""
     T = h.shape[0]
     H, G, D, Dv = m["heads"], m.get("kv_heads") or m["heads"], m["dim"], m["vdim"]
-    q = silu(causal_conv(h @ w("q").T, w("q.conv"))).view(T, G, D)
-    k = silu(causal_conv(h @ w("k").T, w("k.conv"))).view(T, G, D)
-    v = silu(causal_conv(h @ w("v").T, w("v.conv"))).view(T, H, Dv)
+    q = silu(causal_conv(mm(h, w("q")), w("q.conv"))).view(T, G, D)
+    k = silu(causal_conv(mm(h, w("k")), w("k.conv"))).view(T, G, D)
+    v = silu(causal_conv(mm(h, w("v")), w("v.conv"))).view(T, H, Dv)
     q = q / torch.sqrt((q * q).sum(-1, keepdim=True) + 1e-6) * D ** -0.5
     k = k / torch.sqrt((k * k).sum(-1, keepdim=True) + 1e-6)
-    beta = torch.sigmoid(h @ w("b").T)                                         # [T, H]
-    a = (h @ w("a1").T) @ w("a2").T + w("dt_bias")                             # [T, H * D]
+    beta = torch.sigmoid(mm(h, w("b")))                                        # [T, H]
+    a = mm(mm(h, w("a1")), w("a2")) + w("dt_bias")                             # [T, H * D]
     decay = torch.exp(-torch.exp(w("A_log"))[None, :, None] * torch.nn.functional.softplus(a.view(T, H, D)))
-    gate = torch.sigmoid((h @ w("g1").T) @ w("g2").T).view(T, H, Dv)
+    gate = torch.sigmoid(mm(mm(h, w("g1")), w("g2"))).view(T, H, Dv)
     rep = H // G
     out = torch.zeros(T, H, Dv, dtype=F)
     S = torch.zeros(H, D, Dv, dtype=F)
@@ -142,26 +151,47 @@ def channel_delta(h, m, w, eps):
             S[j] = Sj
             out[t, j] = Sj.T @ qt
     out = rms_norm(out, w("norm"), eps) * gate
-    return out.reshape(T, H * Dv) @ w("o").T
+    return mm(out.reshape(T, H * Dv), w("o"))
 
 
 def gated_ff(h, gate, up, down):
-    return (silu(h @ gate.T) * (h @ up.T)) @ down.T
+    return mm(silu(mm(h, gate)) * mm(h, up), down)
+
+
+# every call of `route` leaves here, a token, how far its choice was from another one: the gap between the last
+# chosen and the first unchosen number (experts, and groups), as a fraction of the two rivals' own scores (what moves
+# when the router's input moves is the scores; the corrections stand still)
+route_margins: list = []
+
+
+def _gap(numbers, scores, taken):
+    """[T]: the taken-th largest of numbers [T, n] less the next one, over the sum of the two rivals' scores
+    (infinity where there is no next one, or where the next one cannot be chosen at all)."""
+    if taken >= numbers.shape[1]:
+        return torch.full((numbers.shape[0],), float("inf"), dtype=numbers.dtype)
+    ordered, order = torch.sort(numbers, dim=-1, descending=True)
+    rivals = torch.gather(scores, 1, order[:, taken - 1:taken + 1]).sum(-1)
+    gap = (ordered[:, taken - 1] - ordered[:, taken]) / (rivals + 1e-30)
+    return torch.nan_to_num(gap, nan=float("inf"))
 
 
 def route(h, r, router, correction):
     """-> (chosen [T, top] indices, weights [T, top]) of a softmax router with grouped choice."""
     E = router.shape[0]
-    s = torch.softmax(h @ router.T, dim=-1)
+    s = torch.softmax(mm(h, router), dim=-1)
     choice = s + (correction if correction is not None else 0.0)
     groups = r.get("groups")
+    margin = torch.full((h.shape[0],), float("inf"), dtype=F)
     if groups:
         per = E // groups["count"]
-        best = choice.view(-1, groups["count"], per).max(-1).values
+        best, where = choice.view(-1, groups["count"], per).max(-1)
+        best_scores = torch.gather(s.view(-1, groups["count"], per), 2, where[..., None])[..., 0]
+        margin = _gap(best, best_scores, groups["keep"])
         kept = torch.topk(best, groups["keep"], dim=-1).indices
         allow = torch.zeros_like(best, dtype=torch.bool).scatter_(1, kept, True)
         choice = choice.masked_fill(~allow.repeat_interleave(per, dim=1), float("-inf"))
     chosen = torch.topk(choice, r["top"], dim=-1).indices
+    route_margins.append(torch.minimum(margin, _gap(choice, s, r["top"])))
     return chosen, torch.gather(s, 1, chosen)
 
 
@@ -188,8 +218,8 @@ def feed_forward(h, mlp, w):
 def token_side(x, tokens, i, dim, tensors, eps):
     """The layer's own slice of a second embedding, gated by the residual, projected back and RMS-normed."""
     e = t64(tensors["side.embed"])[tokens][:, i * dim:(i + 1) * dim]
-    g = gelu_tanh(x @ t64(tensors[f"l{i}.side.gate"]).T) * e
-    y = g @ t64(tensors[f"l{i}.side.proj"]).T
+    g = gelu_tanh(mm(x, t64(tensors[f"l{i}.side.gate"]))) * e
+    y = mm(g, t64(tensors[f"l{i}.side.proj"]))
     return rms_norm(y, t64(tensors[f"l{i}.side.norm"]), eps)
 
 
@@ -216,7 +246,7 @@ def forward(config, tensors, tokens, return_layers=False):
             x = x + m * token_side(x, tokens, i, side["dim"], tensors, eps)
         seen.append(x)
     x = layer_norm(x, t64(tensors["final.norm"]), t64(tensors["final.norm.b"]), eps)
-    logits = x @ t64(tensors["head"]).T
+    logits = mm(x, t64(tensors["head"]))
     cap = config.get("logit_softcap")
     if cap:
         logits = cap * torch.tanh(logits / cap)
