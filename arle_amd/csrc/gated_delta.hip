@@ -58,11 +58,12 @@ __global__ __launch_bounds__(kGdThreads) void gated_delta_scan_kernel(
     const int* __restrict__ seg_row0, const int* __restrict__ seg_slot, float* __restrict__ out /* [T, H * Dv] */,
     int H, int G, int D, int Dv) {
   constexpr int DP = kGdParts * DS;   // padded D: what lies past D is zero in LDS and in the registers
-  __shared__ __attribute__((aligned(16))) float q_lds[kGdRows][DP];
-  __shared__ __attribute__((aligned(16))) float k_lds[kGdRows][DP];
-  __shared__ __attribute__((aligned(16))) float g_lds[CHANNEL ? kGdRows : 1][DP];   // CHANNEL: the decays; q_lds then holds g q
-  __shared__ float v_lds[kGdRows][kGdCols];
-  __shared__ float c_lds[kGdRows][4];   // decay (of the head), beta, k . q
+  constexpr int RS = ROWS ? kGdRows : 1;   // rows staged at a time: a decoded row's segment is that one row
+  __shared__ __attribute__((aligned(16))) float q_lds[RS][DP];
+  __shared__ __attribute__((aligned(16))) float k_lds[RS][DP];
+  __shared__ __attribute__((aligned(16))) float g_lds[CHANNEL ? RS : 1][DP];   // CHANNEL: the decays of the key entries
+  __shared__ float v_lds[RS][kGdCols];
+  __shared__ float c_lds[RS][4];   // decay (of the head), beta, k . q
   const int seg = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int lane = tid % kWave, wave = tid / kWave;
   const int kvh = h / (H / G);
@@ -71,7 +72,7 @@ __global__ __launch_bounds__(kGdThreads) void gated_delta_scan_kernel(
   const int col = blockIdx.z * kGdCols + col_in;
   const int part = ROWS ? lane % kGdParts : lane / kGdWaveCols;
   const bool live = col < Dv;
-  const int row0 = seg_row0[seg], rows = seg_row0[seg + 1] - row0;
+  const int row0 = seg_row0[seg], rows = ROWS ? seg_row0[seg + 1] - row0 : 1;
   float* s_ptr = s_state + (static_cast<int64_t>(seg_slot[seg]) * H + h) * D * Dv;
   const float rate = expf(a_log[h]), bias = CHANNEL ? 0.f : dt_bias[h], q_scale = 1.0f / sqrtf(static_cast<float>(D));
 
@@ -84,14 +85,17 @@ __global__ __launch_bounds__(kGdThreads) void gated_delta_scan_kernel(
   // A block's rows are fetched from memory into registers while the chain of the block before runs, and go on to LDS
   // (with their norms and gates) when it has ended.
   constexpr int kMine = DP / kGdRowThreads;                      // entries of a row's q (and k) a thread prepares
-  constexpr int kValues = kGdRows * kGdCols / kGdThreads;        // entries of the block's v a thread moves
+  constexpr int kValues = (RS * kGdCols + kGdThreads - 1) / kGdThreads;   // entries of the block's v a thread moves
   const int r = tid / kGdRowThreads, sub = tid % kGdRowThreads;   // a row by kGdRowThreads threads
   float q_next[kMine], k_next[kMine], v_next[kValues], b_next = 0.f, a_next = 0.f;
-  float g_next[CHANNEL ? kMine : 1], g_bias[CHANNEL ? kMine : 1];   // CHANNEL: a_hd of the row, and dt_bias_hd
+  // CHANNEL: a_hd of the row and dt_bias_hd.  With portions a row's eight threads take the entries they prepare of q
+  // and k; a decoded row's entries go one a thread (entry `tid`), so that the exponentials are one deep, not sixteen.
+  constexpr int kDecays = ROWS ? kMine : 1;
+  float g_next[CHANNEL ? kDecays : 1], g_bias[CHANNEL ? kDecays : 1];
   if constexpr (CHANNEL) {
 #pragma unroll
-    for (int j = 0; j < kMine; ++j) {
-      const int d = sub + j * kGdRowThreads;
+    for (int j = 0; j < kDecays; ++j) {
+      const int d = ROWS ? sub + j * kGdRowThreads : tid;
       g_bias[j] = d < D ? dt_bias[h * D + d] : 0.f;
     }
   }
@@ -106,8 +110,9 @@ __global__ __launch_bounds__(kGdThreads) void gated_delta_scan_kernel(
       const bool there = r < n && d < D;
       q_next[j] = there ? to_float(qr[d]) : 0.f;
       k_next[j] = there ? to_float(kr[d]) : 0.f;
-      if constexpr (CHANNEL) g_next[j] = there ? decay_in[t * decay_stride + h * D + d] : 0.f;
+      if constexpr (CHANNEL && ROWS) g_next[j] = there ? decay_in[t * decay_stride + h * D + d] : 0.f;
     }
+    if constexpr (CHANNEL && !ROWS) g_next[0] = (n > 0 && tid < D) ? decay_in[(row0 + base) * decay_stride + h * D + tid] : 0.f;
     if (sub == 0 && r < n) {
       b_next = beta_in[t * beta_stride + h];
       if constexpr (!CHANNEL) a_next = decay_in[t * decay_stride + h];
@@ -116,7 +121,7 @@ __global__ __launch_bounds__(kGdThreads) void gated_delta_scan_kernel(
     for (int j = 0; j < kValues; ++j) {
       const int e = tid + j * kGdThreads, rr = e / kGdCols, cc = e % kGdCols;
       const int c_abs = min(static_cast<int>(blockIdx.z) * kGdCols + cc, Dv - 1);
-      v_next[j] = rr < n ? to_float(v[(row0 + base + rr) * v_stride + h * Dv + c_abs]) : 0.f;
+      v_next[j] = (rr < n && e < RS * kGdCols) ? to_float(v[(row0 + base + rr) * v_stride + h * Dv + c_abs]) : 0.f;
     }
   };
   fetch(0);
@@ -140,13 +145,9 @@ __global__ __launch_bounds__(kGdThreads) void gated_delta_scan_kernel(
       const float fq = q_scale / sqrtf(sq + unit_eps), fk = 1.0f / sqrtf(sk + unit_eps);
 #pragma unroll
       for (int j = 0; j < kMine; ++j) {
-        if constexpr (CHANNEL) {   // (past D: a decay of 1 on zeros)
-          const float gd = expf(-rate * softplus(g_next[j] + g_bias[j]));
-          g_lds[r][sub + j * kGdRowThreads] = gd;
-          q_lds[r][sub + j * kGdRowThreads] = q_next[j] * fq * gd;
-        } else {
-          q_lds[r][sub + j * kGdRowThreads] = q_next[j] * fq;
-        }
+        if constexpr (CHANNEL && ROWS)   // (past D: some decay on zeros)
+          g_lds[r][sub + j * kGdRowThreads] = expf(-rate * softplus(g_next[j] + g_bias[j]));
+        q_lds[r][sub + j * kGdRowThreads] = q_next[j] * fq;
         k_lds[r][sub + j * kGdRowThreads] = k_next[j] * fk;
       }
       if (sub == 0) {
@@ -155,16 +156,32 @@ __global__ __launch_bounds__(kGdThreads) void gated_delta_scan_kernel(
         c_lds[r][2] = kq * fq * fk;
       }
     }
+    if constexpr (CHANNEL && !ROWS) {
+      if (tid < DP) g_lds[0][tid] = expf(-rate * softplus(g_next[0] + g_bias[0]));
+    }
 #pragma unroll
     for (int j = 0; j < kValues; ++j) {
       const int e = tid + j * kGdThreads;
-      v_lds[e / kGdCols][e % kGdCols] = v_next[j];
+      if (e < RS * kGdCols) v_lds[e / kGdCols][e % kGdCols] = v_next[j];
     }
     __syncthreads();
     fetch(base + kGdRows);
     for (int r = 0; r < n; ++r) {
       const float g = c_lds[r][0], beta = c_lds[r][1], kq = c_lds[r][2];
-      float kk[DS], gg[CHANNEL ? DS : 1], dk = 0.f, dq = 0.f;
+      float kk[DS], dk = 0.f, dq = 0.f;
+      if constexpr (CHANNEL) {   // the decayed state diag(g) S first, in the registers: everything below reads it
+        if constexpr (DS % 4 == 0) {
+          const float4* g4 = reinterpret_cast<const float4*>(&g_lds[r][part * DS]);
+#pragma unroll
+          for (int i = 0; i < DS / 4; ++i) {
+            const float4 gv = g4[i];
+            S[4 * i] *= gv.x; S[4 * i + 1] *= gv.y; S[4 * i + 2] *= gv.z; S[4 * i + 3] *= gv.w;
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < DS; ++i) S[i] *= g_lds[r][part * DS + i];
+        }
+      }
       if constexpr (DS % 4 == 0) {
         const float4* k4 = reinterpret_cast<const float4*>(&k_lds[r][part * DS]);
         const float4* q4 = reinterpret_cast<const float4*>(&q_lds[r][part * DS]);
@@ -172,10 +189,7 @@ __global__ __launch_bounds__(kGdThreads) void gated_delta_scan_kernel(
         for (int i = 0; i < DS / 4; ++i) {
           const float4 kv = k4[i], qv = q4[i];
           kk[4 * i] = kv.x; kk[4 * i + 1] = kv.y; kk[4 * i + 2] = kv.z; kk[4 * i + 3] = kv.w;
-          if constexpr (CHANNEL) {
-            const float4 gv = reinterpret_cast<const float4*>(&g_lds[r][part * DS])[i];
-            gg[4 * i] = gv.x; gg[4 * i + 1] = gv.y; gg[4 * i + 2] = gv.z; gg[4 * i + 3] = gv.w;
-          }
+
           dq = fmaf(S[4 * i], qv.x, dq); dq = fmaf(S[4 * i + 1], qv.y, dq);
           dq = fmaf(S[4 * i + 2], qv.z, dq); dq = fmaf(S[4 * i + 3], qv.w, dq);
         }
@@ -183,14 +197,11 @@ __global__ __launch_bounds__(kGdThreads) void gated_delta_scan_kernel(
 #pragma unroll
         for (int i = 0; i < DS; ++i) {
           kk[i] = k_lds[r][part * DS + i];
-          if constexpr (CHANNEL) gg[i] = g_lds[r][part * DS + i];
           dq = fmaf(S[i], q_lds[r][part * DS + i], dq);
         }
       }
-      // CHANNEL: the decayed state is diag(g) S: its products with k and q are S^T (g k) and S^T (g q), the latter
-      // through q_lds, which holds g q
 #pragma unroll
-      for (int i = 0; i < DS; ++i) dk = fmaf(S[i], CHANNEL ? gg[i] * kk[i] : kk[i], dk);
+      for (int i = 0; i < DS; ++i) dk = fmaf(S[i], kk[i], dk);
       if constexpr (ROWS) {   // over the shares of D: with share p ^ 1, then p ^ 2, p ^ 4, p ^ 8
         dk = row16_sum(dk);
         dq = row16_sum(dq);
@@ -203,7 +214,7 @@ __global__ __launch_bounds__(kGdThreads) void gated_delta_scan_kernel(
       }
       const float u = beta * (v_lds[r][col_in] - g * dk);
 #pragma unroll
-      for (int i = 0; i < DS; ++i) S[i] = fmaf(kk[i], u, (CHANNEL ? gg[i] : g) * S[i]);
+      for (int i = 0; i < DS; ++i) S[i] = fmaf(kk[i], u, CHANNEL ? S[i] : g * S[i]);
       if (part == 0 && live) out[static_cast<int64_t>(row0 + base + r) * (H * Dv) + h * Dv + col] = fmaf(u, kq, g * dq);
     }
   }

@@ -101,17 +101,24 @@ __global__ __launch_bounds__(kPostThreads) void norm_add_kernel(float* __restric
   const float inv = 1.0f / sqrtf(total / static_cast<float>(width) + eps);
   float* res = residual + r * width;
   const float one = one_plus ? 1.0f : 0.0f;
+  const bool plain_add = mult == 1.0f && !bias;
   for (int i = kStep * threadIdx.x; i < width; i += kStep * kPostThreads) {
     if (VEC) {
       const float4 g = ld4<TW>(w + i), y = *reinterpret_cast<const float4*>(ys + i);
       const float4 c = bias ? ld4<TW>(bias + i) : float4{0.f, 0.f, 0.f, 0.f};
       float4 v = *reinterpret_cast<const float4*>(res + i);
-      v.x = fmaf(mult, fmaf(y.x * inv, one + g.x, c.x), v.x); v.y = fmaf(mult, fmaf(y.y * inv, one + g.y, c.y), v.y);
-      v.z = fmaf(mult, fmaf(y.z * inv, one + g.z, c.z), v.z); v.w = fmaf(mult, fmaf(y.w * inv, one + g.w, c.w), v.w);
+      if (plain_add) {   // no factor and no bias: one fused multiply-add an entry, rounded once
+        v.x = fmaf(y.x * inv, one + g.x, v.x); v.y = fmaf(y.y * inv, one + g.y, v.y);
+        v.z = fmaf(y.z * inv, one + g.z, v.z); v.w = fmaf(y.w * inv, one + g.w, v.w);
+      } else {
+        v.x = fmaf(mult, fmaf(y.x * inv, one + g.x, c.x), v.x); v.y = fmaf(mult, fmaf(y.y * inv, one + g.y, c.y), v.y);
+        v.z = fmaf(mult, fmaf(y.z * inv, one + g.z, c.z), v.z); v.w = fmaf(mult, fmaf(y.w * inv, one + g.w, c.w), v.w);
+      }
       *reinterpret_cast<float4*>(res + i) = v;
       if (act) st4<TAct>(act + r * width + i, v);
     } else {
-      const float v = fmaf(mult, fmaf(ys[i] * inv, one + to_float(w[i]), bias ? to_float(bias[i]) : 0.f), res[i]);
+      const float v = plain_add ? fmaf(ys[i] * inv, one + to_float(w[i]), res[i])
+                                : fmaf(mult, fmaf(ys[i] * inv, one + to_float(w[i]), bias ? to_float(bias[i]) : 0.f), res[i]);
       res[i] = v;
       if (act) act[r * width + i] = from_float<TAct>(v);
     }

@@ -6,6 +6,7 @@
     python bench.py --workload gufasun [--shape 4b|8b] [--layers L]  (the Gufasun design beside Qwen3 at equal sizes)
     python bench.py --workload sovutar [--shape 4b|8b] [--layers L]  (the Sovutar design beside Qwen3 at equal sizes)
     python bench.py --workload tazitar [--shape 4b|8b] [--layers L]  (the Tazitar design beside Qwen3 at equal sizes)
+    python bench.py --workload retudra [--shape 4b|8b] [--layers L]  (the Retudra design beside Sovutar and Qwen3 at equal sizes)
 
 A step is one decode step of `batch` requests, each holding a `prompt`-token random prompt
 (prefilled by the engine itself before the clock starts) and growing by one token per step.
@@ -892,6 +893,91 @@ def tazitar_work(raw: dict, q: dict, tokens: int, batch: int, context: int) -> d
     return work
 
 
+# ---- the Retudra design beside Sovutar and Qwen3 at equal sizes ------------------------------------------
+# The widths and head counts of Qwen3-4B / 8B; the layers cycle through the windowed attention that keeps its first
+# keys, the delta rule with a decay a key channel and the gated latent attention (Sovutar's sizes: a latent of 192 and a
+# rotated part of 64); the first layer's feed-forward is dense, the others have sixteen experts and two identity experts
+# in three groups of which two are kept, four choices a token; a token-side input of 256 columns a layer.
+def retudra_config(shape: str, layers: int) -> dict:
+    q, span, ff = SOVUTAR_SHAPES[shape]
+    H, G, D = q["num_attention_heads"], q["num_key_value_heads"], q["head_dim"]
+    attn = {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5, "rot": {"base": 1000000.0, "dims": D // 2},
+            "mask": {"size": span, "keep_first": 64}}
+    lat = {"heads": H, "dim": D, "rot_dim": 64, "vdim": D, "kv_rank": 192, "scale": (D + 64) ** -0.5,
+           "rot": {"base": 1000000.0, "dims": 64}}
+    dlt = {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "conv": 4, "decay_rank": 64, "gate_rank": 64}
+    kinds = [("attention", attn), ("channel_delta", dlt), ("latent_attention", lat)]
+    moe = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": 16, "top": 4, "identity": 2, "groups": {"count": 3, "keep": 2}}}
+    out = [{"type": kinds[i % 3][0], "mixer": json.loads(json.dumps(kinds[i % 3][1])),
+            "mlp": {"kind": "dense", "ff": q["intermediate_size"]} if i == 0 else json.loads(json.dumps(moe))}
+           for i in range(layers)]
+    return {"architecture": "Retudra", "vocab": q["vocab_size"], "width": q["hidden_size"], "norm": {"eps": 1e-6},
+            "residual_mult": 0.5, "token_side": {"dim": 256}, "logit_softcap": 30.0, "layers": out}
+
+
+def retudra_work(raw: dict, q: dict, tokens: int, batch: int, context: int) -> dict:
+    """Ideal work of the design's kernels, per step: kernel family -> (bytes, flops)."""
+    W, L = raw["width"], len(raw["layers"])
+    of = lambda kind: [l for l in raw["layers"] if l["type"] == kind]
+    n_att, n_dlt, n_lat = len(of("attention")), len(of("channel_delta")), len(of("latent_attention"))
+    moes = [l["mlp"] for l in raw["layers"] if l["mlp"] and l["mlp"]["kind"] == "moe"]
+    decode = tokens == batch
+    work = {"token_gate_kernel": (L * tokens * raw["token_side"]["dim"] * 6, 0)}
+    top = moes[0]["router"]["top"] if moes else 0
+    # a norm on a sublayer's output: the addend (32-bit; the experts' `top` outputs), the residual in and out, its rounded copy
+    work["norm_add_kernel"] = (tokens * W * ((2 * L + (L - len(moes))) * 14 + len(moes) * (top * 4 + 10)), 0)
+    if n_att:
+        a = of("attention")[0]["mixer"]
+        H, G, D, Dv, span = a["heads"], a["kv_heads"], a["dim"], a["vdim"], a["mask"]["size"]
+        keys = min(span + a["mask"]["keep_first"], context) if decode else min(span, tokens / 2)
+        work["wide_norm_store_kernel"] = (n_att * tokens * (H * D + G * D + G * Dv) * 4, 0)
+        att_bytes = n_att * batch * keys * G * (D + Dv) * 2 if decode else 0
+        att_flops = n_att * tokens * keys * H * 2 * (D + Dv)
+    else:
+        att_bytes = att_flops = 0
+    if n_lat:
+        m = of("latent_attention")[0]["mixer"]
+        LH, LD, R, LDv, C = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
+        keys = context if decode else tokens / 2
+        att_bytes += n_lat * batch * keys * (2 * C + R) * 2 if decode else 0
+        att_flops += n_lat * tokens * keys * LH * 2 * (2 * C + R)
+        work["latent_prep_kernel"] = (n_lat * tokens * (LH * R * 2 + (C + R) + 2 * C + R) * 2, 0)
+        work["head_proj"] = (n_lat * (tokens * LH * (LD + 2 * C + LDv) * 2 + LH * C * (LD + LDv) * 2),
+                             n_lat * tokens * LH * C * (LD + LDv) * 2)
+        work["gate_mul"] = (n_lat * tokens * LH * LDv * 6, 0)
+    work["attn_softcap_mfma_kernel"] = (att_bytes, att_flops)
+    if n_dlt:
+        r = of("channel_delta")[0]["mixer"]
+        state = r["heads"] * r["dim"] * r["vdim"]
+        conv = 2 * r["kv_heads"] * r["dim"] + r["heads"] * r["vdim"]
+        work.update({"causal_conv": (n_dlt * tokens * conv * 4, 0),
+                     "gated_delta_scan_kernel": (n_dlt * (batch * state * 8 + tokens * r["heads"] * r["dim"] * 4), n_dlt * tokens * state * 8),
+                     "gated_delta_output_kernel": (n_dlt * tokens * r["heads"] * r["vdim"] * 8, 0)})
+    if moes:
+        E, F = moes[0]["router"]["experts"], moes[0]["expert"]["ff"]
+        outputs = E + moes[0]["router"].get("identity", 0)
+        active = min(E, batch * top) if decode else E
+        n = len(moes)
+        work.update({"moe_route_kernel": (n * (tokens + outputs) * W * 2, 0),
+                     "moe_expert": (n * (active * 3 * W * F * 2 + tokens * top * (W * 2 + F * 4 + W * 4)), n * tokens * top * 3 * W * F * 2),
+                     "moe_identity_kernel": (n * tokens * top * W * 6 * moes[0]["router"].get("identity", 0) / outputs, 0)})
+    return work
+
+
+def retudra_bench(args) -> int:
+    """Prefill and decode throughput of the Retudra design, of Sovutar (the closest design: sublayers normed on their
+    way out, a latent attention, a mixture of experts) and of Qwen3 at the same widths and depth."""
+    from arle_amd.config import Qwen3Config, RetudraConfig, SovutarConfig
+
+    layers = args.layers if args.layers != FULL_LAYERS else 8
+    q = dict(SOVUTAR_SHAPES[args.shape][0], num_hidden_layers=layers)
+    raw, sov = retudra_config(args.shape, layers), sovutar_config(args.shape, layers)
+    models = {"retudra": ("Retudra", RetudraConfig.from_dict(raw)), "sovutar": ("Sovutar", SovutarConfig.from_dict(sov)),
+              "qwen3": ("Qwen3ForCausalLM", Qwen3Config.from_dict(q))}
+    return design_bench(args, "retudra", models, q, layers, lambda tokens, batch, context: retudra_work(raw, q, tokens, batch, context),
+                        {"sovutar": lambda tokens, batch, context: sovutar_work(sov, q, tokens, batch, context)})
+
+
 def tazitar_bench(args) -> int:
     """Prefill and decode throughput of the Tazitar design and of Qwen3 at the same widths and depth."""
     from arle_amd.config import Qwen3Config, TazitarConfig
@@ -925,9 +1011,10 @@ def gufasun_bench(args) -> int:
     return design_bench(args, "gufasun", models, q, layers, lambda tokens, batch, context: gufasun_work(raw, q, tokens, batch, context))
 
 
-def design_bench(args, design: str, models: dict, q: dict, layers: int, design_work) -> int:
-    """Prefill and decode throughput of a design and of Qwen3 at the same widths and depth, one JSON line each, and the
-    time of a step by kernel family with what each new kernel reaches of its roofline."""
+def design_bench(args, design: str, models: dict, q: dict, layers: int, design_work, other_work: dict | None = None) -> int:
+    """Prefill and decode throughput of a design and of Qwen3 (and further models) at the same widths and depth, one JSON
+    line each, and the time of a step by kernel family with what each new kernel reaches of its roofline.
+    other_work: {model name: its ideal work} for models beside the design and Qwen3."""
     import torch
 
     from arle_amd.engine import Engine, StepEntry
@@ -983,8 +1070,9 @@ def design_bench(args, design: str, models: dict, q: dict, layers: int, design_w
             t = toks(prompt)
             pre, dec = profiled_steps(torch, [lambda: engine.step([StepEntry("prof", t, [prompt - 1])]), decode_step])
             engine.end_request("prof")
-            work = {"prefill": design_work(prompt, 1, 0) if name == design else qwen3_work(q, layers, prompt, 1, 0),
-                    "decode": design_work(batch, batch, prompt) if name == design else qwen3_work(q, layers, batch, batch, prompt)}
+            ideal = design_work if name == design else (other_work or {}).get(
+                name, lambda tokens, rows, context: qwen3_work(q, layers, tokens, rows, context))
+            work = {"prefill": ideal(prompt, 1, 0), "decode": ideal(batch, batch, prompt)}
             for phase, step in (("prefill", pre), ("decode", dec)):
                 fam: dict = {}
                 for kname, us in step:
@@ -1050,10 +1138,10 @@ def main() -> int:
                          "and write the table that ARLE_AMD_PRODUCT_TABLE / ops.load_product_table reads; WIDTHS: 4b, 8b, "
                          "32b or hidden,q_width,kv_width,intermediate[,vocabulary]")
     ap.add_argument("--out", default=None, help="--tune-products: the table's file (default: product_table_<widths>.json)")
-    ap.add_argument("--workload", default="qwen3-4b", choices=["qwen3-4b", "qwen3-8b-mixed", "qwen3-32b-decode", "gufasun", "sovutar", "tazitar"],
+    ap.add_argument("--workload", default="qwen3-4b", choices=["qwen3-4b", "qwen3-8b-mixed", "qwen3-32b-decode", "gufasun", "sovutar", "tazitar", "retudra"],
                     help="qwen3-4b is the default run; the next two are further workloads at larger shapes; gufasun: "
                          "the Gufasun design beside Qwen3 at equal widths and depth (--shape, --layers, --batch, --prompt-len)")
-    ap.add_argument("--shape", default="4b", choices=["4b", "8b"], help="--workload gufasun / sovutar / tazitar: whose widths")
+    ap.add_argument("--shape", default="4b", choices=["4b", "8b"], help="--workload gufasun / sovutar / tazitar / retudra: whose widths")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for --gpus {args.gpus})")
@@ -1079,6 +1167,8 @@ def main() -> int:
         return sovutar_bench(args)
     if args.workload == "tazitar":
         return tazitar_bench(args)
+    if args.workload == "retudra":
+        return retudra_bench(args)
     if args.workload == "qwen3-4b" and args.batch is None:
         args.batch = 8
     if args.workload != "qwen3-4b":
