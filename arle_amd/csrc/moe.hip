@@ -192,16 +192,22 @@ __global__ __launch_bounds__(kRouteThreads) void moe_route_kernel(const T* __res
 }
 
 // The rows of experts without tensors: where token t's k-th choice is a router output from `first` on, row t * top + k
-// of out (float32 [T * top, width]) is the token's input itself.  One workgroup a (token, choice).
+// of out (float32 [T * top, width]) is the token's input itself.  One workgroup a token: it reads the row once and
+// writes it for each such choice (most tokens have none, and their workgroups leave after reading `top` numbers).
 template <typename T>
 __global__ __launch_bounds__(256) void moe_identity_kernel(const T* __restrict__ x, long long x_stride,
                                                            const int* __restrict__ ids, float* __restrict__ out, int top,
                                                            int width, int first) {
-  const int64_t item = blockIdx.x;
-  if (ids[item] < first) return;
-  const T* row = x + (item / top) * x_stride;
-  float* dst = out + item * width;
-  for (int i = threadIdx.x; i < width; i += 256) dst[i] = to_float(row[i]);
+  const int64_t t = blockIdx.x;
+  unsigned long long which = 0;   // bit k: the k-th choice is such an expert (top <= 64)
+  for (int k = 0; k < top; ++k) which |= static_cast<unsigned long long>(ids[t * top + k] >= first) << k;
+  if (!which) return;
+  const T* row = x + t * x_stride;
+  for (int i = threadIdx.x; i < width; i += 256) {
+    const float v = to_float(row[i]);
+    for (unsigned long long left = which; left; left &= left - 1)
+      out[(t * top + __builtin_ctzll(left)) * width + i] = v;
+  }
 }
 
 constexpr int kEM = 64, kEN = 64, kEK = 16;
@@ -623,9 +629,9 @@ extern "C" int arle_moe_route(const void* x, long long x_stride, int x_dtype, co
 extern "C" int arle_moe_identity(const void* x, long long x_stride, int dtype, const int* ids, void* out, int tokens,
                                  int top, int width, int first, void* stream) {
   if (tokens == 0) return 0;
-  if (top < 1 || width < 1 || first < 0) return static_cast<int>(hipErrorInvalidValue);
+  if (top < 1 || top > 64 || width < 1 || first < 0) return static_cast<int>(hipErrorInvalidValue);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const unsigned items = static_cast<unsigned>(tokens) * top;
+  const unsigned items = static_cast<unsigned>(tokens);
   if (dtype == kF32)
     moe_identity_kernel<float><<<items, 256, 0, s>>>(static_cast<const float*>(x), x_stride, ids, static_cast<float*>(out), top, width, first);
   else
