@@ -195,7 +195,7 @@ ATTENTIONS = [
     (attn(5, 1, 12, 6, scale=0.5), 8, 33, (0, 16)),                                        # no window, no rotation
     (attn(1, None, 10, 14, scale=0.6, rot=rot(20.0, 6), mask=(7, 0)), 8, 30, (22, 23)),      # a window that keeps nothing
     (attn(3, 1, 24, 16, scale=0.3, rot=rot(300.0, 8), mask=(5, 40)), 4, 36, (0, 30)),        # keeps more than it has
-    (attn(4, 2, 64, 64, scale=0.125, rot=rot(500000.0, 32), mask=(40, 18)), 16, 150, (17, 18, 109, 110, 31, 32)),
+    (attn(6, 2, 64, 64, scale=0.125, rot=rot(250000.0, 16), mask=(40, 18)), 16, 150, (17, 18, 109, 110, 31, 32)),
     (attn(2, 1, 128, 64, scale=0.09, rot=rot(800.0, 64), mask=(33, 32)), 16, 120, (31, 32, 86, 87)),
     (attn(8, 2, 64, 32, scale=0.125, rot=rot(1000.0, 64), mask=(16, 16)), 16, 100, (15, 16, 83, 84)),
     (attn(4, 4, 48, 80, scale=0.15, rot=rot(1000.0, 16), mask=(64, 1)), 32, 200, (0, 1, 135, 136)),
@@ -233,7 +233,7 @@ LATENTS = [
     (latent(4, 16, 8, 12, 24, scale=0.3, rot=rot(500.0, 8)), 4, 50),
     (latent(1, 10, 6, 14, 18, scale=0.4, rot=rot(50.0, 4)), 8, 40),          # one head; only part of the rotated part turns
     (latent(4, 32, 32, 48, 64, scale=0.12, rot=rot(250000.0, 32)), 16, 130),
-    (latent(8, 64, 16, 64, 112, scale=0.1, rot=rot(500000.0, 16)), 16, 90),
+    (latent(8, 64, 32, 48, 112, scale=0.1, rot=rot(100000.0, 32)), 16, 90),
     (latent(3, 8, 2, 8, 6, scale=0.5, rot=rot(10.0, 2)), 4, 30),
 ]
 
@@ -258,7 +258,7 @@ def test_the_latent_attention_rotates_halves_and_gates_its_heads(dtype, case):
 DELTAS = [
     (delta(4, 2, 16, 12), 50),
     (delta(3, None, 10, 6, conv=2, decay_rank=3, gate_rank=5), 40),
-    (delta(4, 2, 64, 32, conv=3, decay_rank=16, gate_rank=16), 70),
+    (delta(4, 2, 64, 48, conv=4, decay_rank=16, gate_rank=8), 70),
     (delta(4, 1, 128, 16, conv=5, decay_rank=12, gate_rank=4), 45),
     (delta(2, 1, 130, 20, conv=1, decay_rank=1, gate_rank=1), 37),
     (delta(5, 5, 24, 40, conv=3, decay_rank=7, gate_rank=9), 66),

@@ -8,8 +8,8 @@ Q: what models often make equal differs and what is often large is 1: no token s
    one kv head for five q heads, an attention without window and one without rotation, a window that keeps nothing, a
    delta rule with as many q/k heads as heads and two taps, an expert choice of one among all (no groups, no identity
    experts), sizes that are no multiples of 4 or 8, a latent whose rotated part turns only in its first entries.
-R: sizes the matrix cores take (keys and values of 64, a latent of 64 + 32), pages of 16, a window of 40 that keeps 18
-   (neither a multiple of a tile), seven experts and one identity expert in two groups of which one is kept, three
+R: sizes the matrix cores take (keys and values of 64, three q heads a kv head, a latent of 64 + 32), pages of 16, a
+   window of 40 that keeps 18 (neither a multiple of a tile), seven experts and one identity expert in two groups of which one is kept, three
    choices, a factor of 0.25.
 S: heads of 128 over values of 64, a window of 33 that keeps a whole page of 32, a delta rule with key size 128 and one
    q/k head for four heads, nine router outputs in three groups of which two are kept, five taps.
@@ -84,9 +84,9 @@ TINY_Q = {"architecture": ARCH, "vocab": 97, "width": 42, "norm": {"eps": 1e-6},
 TINY_R = {"architecture": ARCH, "vocab": 300, "width": 96, "norm": {"eps": 1e-5}, "residual_mult": 0.25,
           "token_side": {"dim": 16}, "logit_softcap": 40.0,
           "layers": [layer("latent_attention", latent(4, 32, 32, 48, 64, scale=0.12, rot=rot(250000.0, 32)), dense(128)),
-                     layer("attention", attn(4, 2, 64, 64, scale=0.125, rot=rot(500000.0, 32), mask=(40, 18)),
+                     layer("attention", attn(6, 2, 64, 64, scale=0.125, rot=rot(250000.0, 16), mask=(40, 18)),
                            moe(7, 3, 48, identity=1, groups=(2, 1))),
-                     layer("channel_delta", delta(4, 2, 64, 32, conv=3, decay_rank=16, gate_rank=16),
+                     layer("channel_delta", delta(4, 2, 64, 48, conv=4, decay_rank=16, gate_rank=8),
                            moe(7, 3, 48, identity=1, groups=(2, 1)))]}
 
 TINY_S = {"architecture": ARCH, "vocab": 150, "width": 80, "norm": {"eps": 1e-5}, "residual_mult": 0.7,
