@@ -91,24 +91,27 @@ class GatedDeltaMixer(Part):
         if self.decay not in self.DECAYS or self.gate not in self.GATES:
             raise ValueError(f"decay is one of {self.DECAYS} and gate one of {self.GATES}")
         low_gate = self.gate == "sigmoid_low_rank"
+        channel = self.decay == "channel"
         if low_gate and tensors["g1"].shape[0] != tensors["g2"].shape[1]:
             raise ValueError("the two projections of the output gate do not meet in one width")
-        fused = [tensors[n] for n in ("q", "k", "v", "g1" if low_gate else "g")]
+        if channel and tensors["a1"].shape[0] != tensors["a2"].shape[1]:
+            raise ValueError("the two projections of the decay do not meet in one width")
+        # one product for q, k, v, the output gate (or its narrow middle) and, with a decay a channel, the decay's
+        # narrow middle: all of them operands of what follows, in the activation type
+        fused = [tensors[n] for n in ("q", "k", "v", "g1" if low_gate else "g")] + ([tensors["a1"]] if channel else [])
         if len({t.dtype for t in fused}) != 1:
             raise ValueError("q, k, v and gate projections must be stored in one type")
+        self.gate_width = int(fused[3].shape[0])
+        self.decay_rank = int(tensors["a1"].shape[0]) if channel else 0
         self.qkvg = Linear(torch.cat(fused, dim=0).contiguous(), rt.weight_tiles)
         self.gate_up = Linear(tensors["g2"], rt.weight_tiles) if low_gate else None
         self.gate_act = ops.GATES["sigmoid" if low_gate else "silu"]
         self.conv = ShortConv(torch.cat([tensors[n] for n in ("q_conv", "k_conv", "v_conv")], dim=0).contiguous())
         # beta and the decay enter the recurrence: their projection hands over 32-bit sums whatever the mode.  In
         # bfloat16 it is a product of bfloat16 operands like every projection (rows padded with zeros to whole tiles
-        # of 16 outputs), in float32 the fixed-order 32-bit product.  With a decay a channel the same projection
-        # makes beta and the narrow middle, and a second one (32-bit sums again) the channels' pre-activations.
-        channel = self.decay == "channel"
-        if channel and tensors["a1"].shape[0] != tensors["a2"].shape[1]:
-            raise ValueError("the two projections of the decay do not meet in one width")
-        self.decay_rank = int(tensors["a1"].shape[0]) if channel else 0
-        gates = torch.cat([tensors["b"], tensors["a1" if channel else "a"]], dim=0)
+        # of 16 outputs), in float32 the fixed-order 32-bit product.  With a decay a channel it makes beta alone, and
+        # the second projection of the decay (32-bit sums again) the channels' pre-activations from the narrow middle.
+        gates = tensors["b"] if channel else torch.cat([tensors["b"], tensors["a"]], dim=0)
         if gates.dtype == torch.bfloat16 and not rt.is_f32:
             pad = -gates.shape[0] % 16
             gates = torch.cat([gates, gates.new_zeros((pad, gates.shape[1]))], dim=0) if pad else gates
@@ -133,16 +136,14 @@ class GatedDeltaMixer(Part):
         p = self.qkvg(x)
         y = self.conv(p[:, :2 * qk + vw], batch, cache.get("conv"), silu=True)
         gates = self.gates(x, out_dtype=torch.float32)
+        at = 2 * qk + vw
+        gate, middle = p[:, at:at + self.gate_width], p[:, at + self.gate_width:]
         channel = None
         if self.decay_up is not None:
-            middle = gates[:, self.H:self.H + self.decay_rank]
-            if self.decay_up.weight.dtype == torch.bfloat16:
-                middle = middle.to(torch.bfloat16)     # an operand of a bfloat16 product like any other
             channel = self.decay_up(middle, out_dtype=torch.float32)
         o = ops.gated_delta_scan(y[:, :qk], y[:, qk:2 * qk], y[:, 2 * qk:], gates, self.a_log, self.dt_bias,
                                  cache["S"].state, batch.seg_row0, batch.seg_slot, heads=self.H, kv_heads=self.G,
                                  key_dim=self.D, value_dim=self.Dv, unit_eps=self.unit_eps, channel_decay=channel)
-        gate = p[:, 2 * qk + vw:]
         if self.gate_up is not None:
             gate = self.gate_up(gate)
         z = ops.gated_delta_output(o, gate, self.norm, self.eps, heads=self.H, value_dim=self.Dv, act=self.gate_act)
